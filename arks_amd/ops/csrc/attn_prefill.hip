@@ -80,8 +80,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   // 32-lane ds_read_b64_tr_b16 group land on disjoint bank halves
   // (stride 192 B = 48 dwords; probe: gpurun_out/probe_layouts.log).
   // Each lane then receives the 4 keys of its column — B-fragment shape —
-  // and V staging becomes two b128 stores instead of 16 scalar b16 writes
-  // (the hot block of the v2 disassembly).
+  // and V staging becomes two b128 stores instead of 16 scalar b16 writes.
   __shared__ __attribute__((aligned(16))) bf16 vt_img[2][HEAD_DIM / 16][8][96];
   __shared__ __attribute__((aligned(16))) bf16 p_lds[NUM_WAVES][QTILE_WAVE][VT_PAD];
 
