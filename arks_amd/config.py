@@ -136,13 +136,103 @@ class ModelConfig:
         )
 
     @classmethod
-    def from_pretrained(cls, model_path: str) -> "ModelConfig":
+    def from_pretrained(cls, model_path: str):
         with open(os.path.join(model_path, "config.json")) as f:
-            return cls.from_hf_config(json.load(f))
+            cfg = json.load(f)
+        if HybridModelConfig.matches(cfg):
+            return HybridModelConfig.from_dict(cfg)
+        return cls.from_hf_config(cfg)
 
     @property
     def num_qo_heads(self) -> int:
         return self.num_attention_heads
+
+
+@dataclass
+class HybridModelConfig:
+    """Layer-list decoders: config.json names one architecture and lists the
+    layers, each with its mixer type ("attention", "lightning", "mamba1"),
+    the mixer's sizes and an optional feed-forward. Every size and every
+    per-model constant comes from that file; what the architecture itself
+    fixes (block arrangement, activation, rotary pairing) lives with the
+    model code (arks_amd/models/hybrid.py)."""
+
+    architecture: str = "Gagorax"
+    vocab_size: int = 512
+    hidden_size: int = 256
+    layers: list = None  # [{"type", "mixer": {...}, "mlp": {...}|None}]
+    rms_norm_eps: float = 1e-5
+    logit_scale: float = 1.0
+    eos_token_id: int = -1  # the format defines no end token
+    bos_token_id: int = -1
+    torch_dtype: str = "bfloat16"
+
+    # what the engine asks of any model config
+    num_local_experts = 0
+    sliding_window = None
+
+    ARCHITECTURES = ("Gagorax",)
+
+    @classmethod
+    def matches(cls, cfg: dict) -> bool:
+        return cfg.get("architecture") in cls.ARCHITECTURES
+
+    @classmethod
+    def from_dict(cls, cfg: dict) -> "HybridModelConfig":
+        layers = []
+        for entry in cfg["layers"]:
+            mlp = entry.get("mlp")
+            if mlp is not None and mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"unknown feed-forward kind {mlp.get('kind')!r}")
+            layers.append({"type": entry["type"], "mixer": dict(entry["mixer"]),
+                           "mlp": dict(mlp) if mlp is not None else None})
+        return cls(
+            architecture=cfg["architecture"],
+            vocab_size=int(cfg["vocab"]),
+            hidden_size=int(cfg["width"]),
+            layers=layers,
+            rms_norm_eps=float(cfg["norm"]["eps"]),
+            logit_scale=float(cfg.get("logit_scale", 1.0)),
+            eos_token_id=int(cfg.get("eos_token_id", -1)),
+            bos_token_id=int(cfg.get("bos_token_id", -1)),
+        )
+
+    def to_dict(self) -> dict:
+        return {"architecture": self.architecture, "vocab": self.vocab_size,
+                "width": self.hidden_size, "layers": self.layers,
+                "norm": {"eps": self.rms_norm_eps},
+                "logit_scale": self.logit_scale}
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    def uniform_window(self) -> int:
+        return 0  # no layer of these designs drops KV pages
+
+
+def _gagorax_preset(width, vocab, pattern, heads, kv_heads, dim, ff,
+                    inner, state, dt_rank, l_heads, l_dim) -> HybridModelConfig:
+    """pattern: string of a (attention), l (lightning), m (mamba1); attention
+    layers carry the feed-forward, as a typical model of the design does."""
+    layers = []
+    for ch in pattern:
+        if ch == "a":
+            layers.append({"type": "attention", "mixer": {
+                "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
+                "rot": {"base": 10000.0, "dims": dim},
+                "scale": dim ** -0.5}, "mlp": {"kind": "dense", "ff": ff}})
+        elif ch == "l":
+            layers.append({"type": "lightning", "mixer": {
+                "heads": l_heads, "dim": l_dim, "vdim": l_dim,
+                "decay": [1.0 - 2.0 ** (-2 - 6 * h / max(l_heads - 1, 1))
+                          for h in range(l_heads)]}, "mlp": None})
+        else:
+            layers.append({"type": "mamba1", "mixer": {
+                "inner": inner, "state": state, "dt_rank": dt_rank,
+                "conv": 4}, "mlp": None})
+    return HybridModelConfig(vocab_size=vocab, hidden_size=width, layers=layers,
+                             rms_norm_eps=1e-5, logit_scale=1.0)
 
 
 # Named synthetic configs for benchmarks / tests (random-init weights; no
@@ -414,6 +504,12 @@ PRESET_CONFIGS: dict[str, ModelConfig] = {
         eos_token_id=2,
         bos_token_id=1,
     ),
+    # Gagorax at the layer sizes of an ~8B dense model (32 layers' worth of
+    # width; 8 layers so one GPU bench run stays short)
+    "gagorax-8b-slice": _gagorax_preset(
+        4096, 32000, "almmalmm", 32, 8, 128, 14336, 8192, 16, 256, 32, 128),
+    "tiny-gagorax": _gagorax_preset(
+        128, 512, "alma", 4, 2, 32, 192, 160, 8, 12, 2, 16),
     "tiny-gpu": ModelConfig(  # GPU-test-sized (head_dim 128 kernels)
         architecture="Qwen2ForCausalLM",
         vocab_size=2048,

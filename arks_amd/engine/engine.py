@@ -29,6 +29,14 @@ class LLMEngine:
         if self.window and cfg.enable_prefix_caching:
             cfg.enable_prefix_caching = False
         self.runner = ModelRunner(cfg, self.model_cfg)
+        if self.runner.seq_state:
+            # per-sequence recurrent state: cached pages alone cannot resume
+            # a prefix, and a verify pass cannot be rolled back
+            cfg.enable_prefix_caching = False
+            if cfg.speculative:
+                raise ValueError(
+                    "speculative decoding is not implemented for models "
+                    f"with recurrent state ({self.model_cfg.architecture})")
         t0 = time.time()
         self.runner.load_weights()
         self.load_seconds = time.time() - t0
@@ -39,6 +47,7 @@ class LLMEngine:
             max_num_batched_tokens=cfg.max_num_batched_tokens,
             max_model_len=cfg.max_model_len,
             mixed_batching=cfg.enable_mixed_batching,
+            state_slots=self.runner.state_slots,
         )
         # serving metrics
         self.total_prompt_tokens = 0

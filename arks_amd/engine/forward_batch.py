@@ -25,6 +25,16 @@ class ForwardBatch:
     # rows of the hidden states from which logits are needed (last token of
     # each sequence for prefill; everything for decode)
     logits_indices: torch.Tensor | None = None
+    # models with per-sequence state (recurrent mixers, token shift): the
+    # slot of every sequence in the slot-addressed state tensors (-1 =
+    # padding row), each row's sequence index, and the longest run of rows
+    # of one sequence (host int, sizes the kernels' grids). For these
+    # models cu_seqlens / seq_lens / block_tables are set for decode
+    # batches too, so one set of kernels serves prompt portions, single
+    # tokens and mixes of both.
+    state_slots: torch.Tensor | None = None  # [num_seqs] int32
+    token_seq: torch.Tensor | None = None  # [total_tokens] int32
+    max_q_len: int = 0
 
     @property
     def num_tokens(self) -> int:

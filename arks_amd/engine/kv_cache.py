@@ -59,6 +59,30 @@ class BlockAllocator:
         return (num_tokens + block_size - 1) // block_size
 
 
+class StateSlotAllocator:
+    """Rows of the slot-addressed state tensors (recurrent state, token
+    shift, conv history): one per live sequence, taken at admission and
+    given back with the pages. Slots are not cleared on reuse — a sequence
+    that starts at position 0 reads zeros instead of its slot."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free: list[int] = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def allocate(self) -> int:
+        if not self._free:
+            raise RuntimeError("no free state slot")
+        return self._free.pop()
+
+    def free(self, slot: int) -> None:
+        assert 0 <= slot < self.num_slots and slot not in self._free, slot
+        self._free.append(slot)
+
+
 class PrefixCachingAllocator(BlockAllocator):
     def __init__(self, num_blocks: int, block_size: int = 16):
         self.num_blocks = num_blocks

@@ -20,7 +20,8 @@ from .. import ops
 from ..config import EngineConfig, ModelConfig
 from ..parallel.comm import get_tp_rank, get_tp_world_size, tp_all_gather
 from .forward_batch import ForwardBatch
-from .kv_cache import BlockAllocator, PrefixCachingAllocator, kv_cache_block_bytes
+from .kv_cache import (BlockAllocator, PrefixCachingAllocator,
+                       StateSlotAllocator, kv_cache_block_bytes)
 from .scheduler import ScheduledBatch
 from .sequence import Sequence
 
@@ -40,12 +41,29 @@ class ModelRunner:
             engine_cfg.device if torch.cuda.is_available() or engine_cfg.device == "cpu"
             else "cpu"
         )
-        self.dtype = torch.bfloat16
+        if engine_cfg.dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"unknown dtype {engine_cfg.dtype!r}")
+        # float32: true 32-bit everywhere (no reduced-precision matmul mode),
+        # for the models that implement it
+        self.dtype = (torch.float32 if engine_cfg.dtype == "float32"
+                      else torch.bfloat16)
+        if self.dtype == torch.float32:
+            torch.backends.cuda.matmul.allow_tf32 = False
+            torch.backends.cudnn.allow_tf32 = False
         torch.manual_seed(engine_cfg.seed)
         self._setup_tunableop()
         from ..models import create_model  # lazy: breaks the import cycle
 
         self.model = create_model(self.model_cfg, dtype=self.dtype)
+        if (self.dtype == torch.float32
+                and not getattr(self.model, "supports_float32", False)):
+            # their GPU kernels take bf16 rows only
+            raise ValueError(
+                f"{self.model_cfg.architecture} is served in bfloat16 only")
+        # models with per-sequence state (recurrent mixers, token shift)
+        # keep it in slot-addressed tensors beside the paged KV
+        self.seq_state = bool(getattr(self.model, "has_sequence_state", False))
+        self.state_slots: StateSlotAllocator | None = None
         self._weights_loaded = False
         self.kv_caches: list[tuple[torch.Tensor, torch.Tensor]] = []
         self.num_blocks = 0
@@ -85,6 +103,10 @@ class ModelRunner:
             from ..loader.safetensors_loader import load_model_weights
 
             load_model_weights(self.model, self.cfg.model_path, self.device)
+            if hasattr(self.model, "missing_tensors"):
+                missing = self.model.missing_tensors()
+                if missing:
+                    raise ValueError(f"checkpoint lacks tensors: {missing[:8]}")
         else:
             # move first so random-init generates directly on the GPU
             self.model.to(self.device)
@@ -106,16 +128,22 @@ class ModelRunner:
             return self.cfg.kv_cache_blocks
         mc = self.model_cfg
         tp = get_tp_world_size()
-        block_bytes = kv_cache_block_bytes(
-            mc.num_hidden_layers,
-            max(mc.num_key_value_heads // tp, 1),
-            mc.head_dim,
-            self.cfg.block_size,
-            dtype_bytes=1 if self.cfg.kv_cache_dtype == "fp8" else 2,
-        )
+        state_bytes = 0
+        if self.seq_state:
+            block_bytes = self.model.kv_block_bytes(self.cfg.block_size)
+            state_bytes = self.model.state_slot_bytes() * self.cfg.max_num_seqs
+        else:
+            block_bytes = kv_cache_block_bytes(
+                mc.num_hidden_layers,
+                max(mc.num_key_value_heads // tp, 1),
+                mc.head_dim,
+                self.cfg.block_size,
+                dtype_bytes=1 if self.cfg.kv_cache_dtype == "fp8" else 2,
+            )
         if self.device.type == "cuda":
             free, total = torch.cuda.mem_get_info(self.device)
             budget = int(total * self.cfg.gpu_memory_utilization) - (total - free)
+            budget -= state_bytes
             budget = max(budget, 2 * block_bytes)
         else:
             budget = 64 * 1024 * 1024  # CPU tests: small pool
@@ -126,6 +154,18 @@ class ModelRunner:
         mc = self.model_cfg
         tp = get_tp_world_size()
         self.num_blocks = self.profile_num_blocks()
+        if self.seq_state:
+            if self.cfg.kv_cache_dtype != "auto" or self.cfg.quantization:
+                raise ValueError("fp8 KV / weights are not implemented for "
+                                 f"{mc.architecture}")
+            self.kv_caches = self.model.allocate_cache(
+                self.num_blocks, self.cfg.block_size, self.cfg.max_num_seqs,
+                self.device)
+            self.state_slots = StateSlotAllocator(self.cfg.max_num_seqs)
+            if self.use_graphs:
+                self._init_graph_buffers()
+            # recurrent state cannot be resumed from cached pages
+            return BlockAllocator(self.num_blocks, self.cfg.block_size)
         nkv = max(mc.num_key_value_heads // tp, 1)
         shape = (self.num_blocks, nkv, self.cfg.block_size, mc.head_dim)
         kv_dtype = (
@@ -152,6 +192,10 @@ class ModelRunner:
         transfer to a decode instance (the reference's PD
         split delegates this to SGLang's disaggregation-mode, reference
         arksdisaggregatedapplication_controller.go:1672-1724)."""
+        if self.seq_state:
+            raise NotImplementedError(
+                "prefill/decode disaggregation does not move per-sequence "
+                "state yet")
         # sliding-window-dropped pages are -1: clamp to a valid page (the
         # receiver never reads out-of-window content)
         bt = torch.tensor(block_table, dtype=torch.long,
@@ -193,7 +237,7 @@ class ModelRunner:
             # the contiguous-varlen kernel is slower and pages are written
             # either way); the CPU reference keeps the contiguous path
             # exercised for fresh prefills.
-            use_extend = (self.device.type == "cuda"
+            use_extend = (self.device.type == "cuda" or self.seq_state
                           or any(s.num_cached_tokens > 0 for s in sb.seqs))
             input_ids: list = []  # np.int64 arrays, one per seq
             positions: list = []
@@ -259,6 +303,7 @@ class ModelRunner:
                     )
                 block_tables = bt.to(dev)
                 seq_lens = torch.tensor(kv_lens, dtype=torch.int32, device=dev)
+            if use_extend and not self.seq_state:
                 ext_tiles = ops.build_extend_tiles(
                     q_lens, kv_lens,
                     self.cfg.kv_cache_dtype == "fp8", dev,
@@ -277,6 +322,7 @@ class ModelRunner:
                 seq_lens=seq_lens,
                 ext_tiles=ext_tiles,
                 logits_indices=torch.tensor(logits_idx, dtype=torch.int64, device=dev),
+                **self._state_fields(sb.seqs, q_lens),
             )
         # decode
         input_ids = [s.last_token() for s in sb.seqs]
@@ -301,6 +347,25 @@ class ModelRunner:
             slot_mapping=torch.tensor(slot_mapping, dtype=torch.int64, device=dev),
             block_tables=bt.to(dev),
             seq_lens=torch.tensor(seq_lens, dtype=torch.int32, device=dev),
+            **(dict(cu_seqlens=torch.arange(len(sb.seqs) + 1, dtype=torch.int32,
+                                            device=dev),
+                    **self._state_fields(sb.seqs, [1] * len(sb.seqs)))
+               if self.seq_state else {}),
+        )
+
+    def _state_fields(self, seqs: list[Sequence], q_lens: list[int]) -> dict:
+        """ForwardBatch fields of models with per-sequence state."""
+        if not self.seq_state:
+            return {}
+        import numpy as np
+
+        dev = self.device
+        return dict(
+            state_slots=torch.tensor([s.state_slot for s in seqs],
+                                     dtype=torch.int32, device=dev),
+            token_seq=torch.from_numpy(np.repeat(
+                np.arange(len(seqs), dtype=np.int32), q_lens)).to(dev),
+            max_q_len=max(q_lens),
         )
 
     # ---------------- hipGraph decode ----------------
@@ -330,7 +395,16 @@ class ModelRunner:
             "h_block_tables": torch.zeros(self._bmax, mb, dtype=torch.int32, pin_memory=True),
             "h_seq_lens": torch.ones(self._bmax, dtype=torch.int32, pin_memory=True),
         }
-        for name in ("input_ids", "positions", "slot_mapping", "block_tables", "seq_lens"):
+        if self.seq_state:
+            self._graph_bufs.update({
+                "state_slots": torch.full((self._bmax,), -1, dtype=torch.int32, device=dev),
+                "h_state_slots": torch.full((self._bmax,), -1, dtype=torch.int32, pin_memory=True),
+                # constants: one row per sequence
+                "cu_seqlens": torch.arange(self._bmax + 1, dtype=torch.int32, device=dev),
+                "token_seq": torch.arange(self._bmax, dtype=torch.int32, device=dev),
+            })
+        for name in ("input_ids", "positions", "slot_mapping", "block_tables",
+                     "seq_lens") + (("state_slots",) if self.seq_state else ()):
             self._graph_bufs["np_" + name] = self._graph_bufs["h_" + name].numpy()
 
     def _capture(self, bs: int) -> "_DecodeGraph":
@@ -343,6 +417,17 @@ class ModelRunner:
             block_tables=b["block_tables"][:bs],
             seq_lens=b["seq_lens"][:bs],
         )
+        if self.seq_state:
+            # warmup and capture run the model for real: every row is made a
+            # padding row first (no cache write, no state slot), or live
+            # sequences' recurrent state would advance
+            b["slot_mapping"][:bs].fill_(-1)
+            b["state_slots"][:bs].fill_(-1)
+            b["seq_lens"][:bs].fill_(1)
+            fb.state_slots = b["state_slots"][:bs]
+            fb.cu_seqlens = b["cu_seqlens"][:bs + 1]
+            fb.token_seq = b["token_seq"][:bs]
+            fb.max_q_len = 1
         # warmup (materializes workspaces outside the graph)
         self.model(fb, self.kv_caches)
         torch.cuda.synchronize(self.device)
@@ -358,6 +443,8 @@ class ModelRunner:
             self._graph_pool = g.pool()
         return _DecodeGraph(graph=g, logits=logits, batch_size=bs)
 
+    _staging_event = None
+
     def _graph_decode(self, sb: ScheduledBatch) -> torch.Tensor:
         B = len(sb.seqs)
         bs = next(s for s in self.GRAPH_SIZES if s >= B)
@@ -367,6 +454,11 @@ class ModelRunner:
         bsz = self.cfg.block_size
         # numpy views of the pinned staging buffers: scalar stores are ~50x
         # cheaper than torch indexed assignment on the decode hot path
+        # the pinned staging buffers are reused every step: the previous
+        # step's async uploads must have left them before they are rewritten
+        # (a caller that does not read that step's logits never syncs)
+        if self._staging_event is not None:
+            self._staging_event.synchronize()
         np_ids = b["np_input_ids"]
         np_pos = b["np_positions"]
         np_slot = b["np_slot_mapping"]
@@ -381,6 +473,11 @@ class ModelRunner:
             bt = seq.block_table
             np_bt[i, : len(bt)] = bt
             seq.num_cached_tokens = seq.num_tokens
+            if self.seq_state:
+                b["np_state_slots"][i] = seq.state_slot
+        if self.seq_state:
+            b["np_state_slots"][B:bs] = -1
+            b["state_slots"][:bs].copy_(b["h_state_slots"][:bs], non_blocking=True)
         if B < bs:  # neutralize padding rows
             np_ids[B:bs] = 0
             np_pos[B:bs] = 0
@@ -390,6 +487,9 @@ class ModelRunner:
         for name in ("input_ids", "positions", "slot_mapping", "seq_lens"):
             b[name][:bs].copy_(b["h_" + name][:bs], non_blocking=True)
         b["block_tables"][:bs].copy_(b["h_block_tables"][:bs], non_blocking=True)
+        if self._staging_event is None:
+            self._staging_event = torch.cuda.Event()
+        self._staging_event.record()
         gr = self._graphs[bs]
         gr.graph.replay()
         return gr.logits[:B]
@@ -398,19 +498,33 @@ class ModelRunner:
     @torch.no_grad()
     def execute(self, sb: ScheduledBatch) -> list[int]:
         """Run one forward + sampling; returns one new token id per seq."""
+        return self.sample(self.forward_logits(sb), sb.seqs)
+
+    @torch.no_grad()
+    def forward_logits(self, sb: ScheduledBatch,
+                       logits_rows: list[int] | None = None) -> torch.Tensor:
+        """One forward over a scheduled batch: [num_seqs, vocab] logits of
+        each sequence's last row, or, with logits_rows (row indices into the
+        batch's packed new tokens), those rows' logits instead."""
         if (
             not sb.is_prefill
             and self.use_graphs
             and self._graph_bufs is not None
             and len(sb.seqs) <= self._bmax
+            and (logits_rows is None or len(logits_rows) == len(sb.seqs))
         ):
-            logits = self._graph_decode(sb)
-            return self.sample(logits, sb.seqs)
+            # decode rows are one per sequence: all of them or none
+            return self._graph_decode(sb)
         fb = self.prepare_batch(sb)
+        if logits_rows is not None:
+            self._lp_prefill = None
+            fb.logits_indices = torch.tensor(logits_rows, dtype=torch.int64,
+                                             device=self.device)
+            return self.model(fb, self.kv_caches)
         logits = self.model(fb, self.kv_caches)  # [num_seqs, vocab]
         if sb.is_prefill and self._lp_prefill is not None:
             logits = self._finish_prompt_logprobs(logits, sb)
-        return self.sample(logits, sb.seqs)
+        return logits
 
     _lp_prefill: tuple | None = None
 
@@ -546,6 +660,8 @@ class ModelRunner:
             logits = self._apply_bias_min_tokens(logits, seqs)
         if any(s.sampling.has_penalties for s in seqs):
             logits = self._apply_penalties(logits, seqs)
+        if logits.is_cuda and logits.dtype != torch.bfloat16:
+            logits = logits.to(torch.bfloat16)  # the sampling kernels' input
         temps = [s.sampling.temperature for s in seqs]
         if all(t == 0.0 for t in temps):
             ids = ops.greedy_sample(logits.contiguous())

@@ -15,7 +15,7 @@ from __future__ import annotations
 from collections import deque
 from dataclasses import dataclass, field
 
-from .kv_cache import BlockAllocator
+from .kv_cache import BlockAllocator, StateSlotAllocator
 from .sequence import Sequence, SeqStatus
 
 
@@ -40,8 +40,12 @@ class Scheduler:
         max_num_batched_tokens: int = 8192,
         max_model_len: int = 8192,
         mixed_batching: bool = True,
+        state_slots: StateSlotAllocator | None = None,
     ):
         self.allocator = allocator
+        # models with per-sequence state: a sequence holds one slot from
+        # admission to release (preemption gives it back and recomputes)
+        self.state_slots = state_slots
         self.max_num_seqs = max_num_seqs
         self.max_num_batched_tokens = max_num_batched_tokens
         self.max_model_len = max_model_len
@@ -124,6 +128,51 @@ class Scheduler:
             return batch
         return self._schedule_decode()
 
+    def schedule_plan(self, plan: list[tuple[Sequence, int]]) -> ScheduledBatch:
+        """One step whose composition is given from outside (replaying a
+        recorded trace): run exactly `n` new tokens of every listed
+        sequence, together. Pages and state slots come from the same
+        allocators as in schedule(); a sequence seen for the first time is
+        admitted here. Only single next tokens of running sequences make a
+        decode batch, anything else runs as a mixed batch — the split
+        schedule() makes."""
+        bs = self.allocator.block_size
+        for seq, n in plan:
+            assert 0 < n <= seq.num_tokens - seq.num_cached_tokens, (
+                seq.request_id, n, seq.num_tokens, seq.num_cached_tokens)
+            if seq.status is SeqStatus.WAITING and seq.state_slot < 0:
+                if len(self.running) >= self.max_num_seqs:
+                    raise RuntimeError("more live sequences than max_num_seqs")
+            need = (BlockAllocator.blocks_needed(seq.num_cached_tokens + n, bs)
+                    - len(seq.block_table))
+            if need > 0:
+                if not self.allocator.can_allocate(need):
+                    raise RuntimeError("KV cache exhausted by the given plan")
+                seq.block_table.extend(self.allocator.allocate(need))
+            if self.state_slots is not None and seq.state_slot < 0:
+                seq.state_slot = self.state_slots.allocate()
+        decode = all(
+            n == 1 and s.status is SeqStatus.RUNNING
+            and s.num_cached_tokens == s.num_tokens - 1 and s.num_tokens > 1
+            for s, n in plan)
+        for seq, n in plan:
+            if (seq.status is SeqStatus.WAITING
+                    and seq.num_cached_tokens + n == seq.num_tokens):
+                self.waiting.remove(seq)
+                seq.status = SeqStatus.RUNNING
+                self.running.append(seq)
+        return ScheduledBatch(seqs=[s for s, _ in plan], is_prefill=not decode,
+                              num_new_tokens=[n for _, n in plan])
+
+    def finish(self, seq: Sequence) -> None:
+        """Give back what a sequence holds (its request is over)."""
+        seq.status = SeqStatus.FINISHED
+        if seq in self.running:
+            self.running.remove(seq)
+        elif seq in self.waiting:
+            self.waiting.remove(seq)
+        self._release(seq)
+
     def _schedule_prefill(self, budget: int | None = None) -> ScheduledBatch | None:
         seqs: list[Sequence] = []
         ntoks: list[int] = []
@@ -136,6 +185,9 @@ class Scheduler:
             n = seq.num_tokens
             toks = seq.all_token_ids
             if len(self.running) + len(seqs) >= self.max_num_seqs:
+                break
+            if (self.state_slots is not None and seq.state_slot < 0
+                    and self.state_slots.num_free == 0):
                 break
             if not seq.block_table:
                 # Fresh admission: reuse cached full blocks of the prompt
@@ -170,6 +222,8 @@ class Scheduler:
                 seq.block_table = reused + seq.block_table
             if need > 0:
                 seq.block_table.extend(self.allocator.allocate(need))
+            if self.state_slots is not None and seq.state_slot < 0:
+                seq.state_slot = self.state_slots.allocate()
             self.allocator.register_prefix(
                 toks[:covered], seq.block_table, len(reused)
             )
@@ -241,6 +295,9 @@ class Scheduler:
             self.allocator.free(seq.block_table)
             seq.block_table = []
         seq._draft_len = 0  # draft-model KV mirror follows the pages
+        if self.state_slots is not None and seq.state_slot >= 0:
+            self.state_slots.free(seq.state_slot)
+            seq.state_slot = -1
 
     def free_finished(self) -> None:
         for seq in self.running:

@@ -59,6 +59,9 @@ class Sequence:
         self.sampling = sampling or SamplingParams()
         self.status = SeqStatus.WAITING
         self.block_table: list[int] = []
+        # row of the slot-addressed state tensors (models with per-sequence
+        # state); -1 = none held
+        self.state_slot = -1
         # Disaggregated prefill: keep KV pages allocated after finish so the
         # decode instance can pull them (scheduler.held).
         self.hold_pages = False

@@ -3,6 +3,7 @@
 from __future__ import annotations
 
 from ..config import ModelConfig
+from .hybrid import HybridForCausalLM
 from .llama_family import LlamaFamilyForCausalLM
 
 _REGISTRY = {
@@ -17,10 +18,13 @@ _REGISTRY = {
     "Qwen2MoeForCausalLM": LlamaFamilyForCausalLM,  # MoE + shared expert
     # llama arch + NoPE every no_rope_layer_interval-th layer + tied embeds
     "SmolLM3ForCausalLM": LlamaFamilyForCausalLM,
+    # layer-list decoder: attention / lightning / mamba1 mixers, fp32
+    # residual, token shift + gated residual (models/hybrid.py)
+    "Gagorax": HybridForCausalLM,
 }
 
 
-def create_model(cfg: ModelConfig, dtype=None):
+def create_model(cfg, dtype=None):
     import torch
 
     cls = _REGISTRY.get(cfg.architecture)

@@ -1,0 +1,245 @@
+"""Layer-list decoders (config.HybridModelConfig): a stack of blocks, each
+with one mixer of arks_amd/models/mixers.py and an optional dense
+feed-forward, around an fp32 residual stream.
+
+What an architecture fixes is a BlockArrangement; Gagorax's is:
+  - the sublayers read the residual x itself and the RMS norm sits on each
+    sublayer's OUTPUT:  x += norm(sublayer(x)) * w
+  - token shift: the mixer reads x_t + (x_{t-1} - x_t) * s (x_{-1} = 0);
+    the last row of every step is per-sequence state in every block
+  - gated residual: the sublayer's result is multiplied by
+    sigmoid(W_g x + b_g) (x unshifted) before that norm
+  - feed-forward = W_down gelu_tanh(W_up x); logits = head(norm(x)) * scale
+
+Kernel plan per block (bf16 serving; fp32 runs the same kernels on float
+rows): token_shift -> GEMM(mixer in) .. mixer kernels .. GEMM(mixer out),
+GEMM(gate) -> gated_norm_residual [-> GEMM(up|gate) -> gelu_tanh ->
+GEMM(down) -> gated_norm_residual]. The feed-forward's up projection and
+its residual gate read the same row, so they are one fused GEMM.
+
+The per-layer cache is a dict of tensors (paged KV for attention, slot
+state for the recurrent mixers and the token shift), allocated by
+allocate_cache() from each mixer's cache_layout(). A sequence that starts at
+position 0 ignores whatever its slot holds, so slots and pages are reused
+without clearing. Tensor parallelism is not implemented for these models.
+"""
+
+from __future__ import annotations
+
+import zlib
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+
+from .. import ops
+from ..config import HybridModelConfig
+from ..engine.forward_batch import ForwardBatch
+from ..parallel.comm import get_tp_world_size
+from .mixers import build_mixer, linear, _param
+
+
+@dataclass(frozen=True)
+class BlockArrangement:
+    token_shift: bool = True
+    gated_residual: bool = True
+    norm_place: str = "output"  # only sublayer-output norms so far
+
+
+ARRANGEMENTS = {"Gagorax": BlockArrangement()}
+
+
+class HybridBlock(nn.Module):
+    def __init__(self, width: int, spec: dict, eps: float, dtype,
+                 arr: BlockArrangement):
+        super().__init__()
+        if arr.norm_place != "output":
+            raise NotImplementedError(arr.norm_place)
+        f32 = torch.float32
+        self.arr, self.eps, self.width = arr, eps, width
+        self.mixer = build_mixer(spec["type"], spec["mixer"], width, eps, dtype)
+        self.norm1 = _param(width, dtype=f32)
+        self.shift = _param(width, dtype=f32) if arr.token_shift else None
+        self.rg1 = _param(width, width, dtype=dtype) if arr.gated_residual else None
+        self.rg1_b = _param(width, dtype=f32) if arr.gated_residual else None
+        self.ff = spec["mlp"]["ff"] if spec.get("mlp") is not None else 0
+        if self.ff:
+            gate_rows = width if arr.gated_residual else 0
+            self.norm2 = _param(width, dtype=f32)
+            self.up_gate = _param(self.ff + gate_rows, width, dtype=dtype)
+            self.down = _param(width, self.ff, dtype=dtype)
+            self.rg2_b = _param(width, dtype=f32) if arr.gated_residual else None
+
+    def weight_map(self) -> dict:
+        m = {"mix." + k: v for k, v in self.mixer.weight_map().items()}
+        m["norm1"] = (self.norm1, 0)
+        if self.shift is not None:
+            m["shift"] = (self.shift, 0)
+        if self.rg1 is not None:
+            m["rg1"] = (self.rg1, 0)
+            m["rg1.b"] = (self.rg1_b, 0)
+        if self.ff:
+            m["norm2"] = (self.norm2, 0)
+            m["mlp.up"] = (self.up_gate, 0)
+            m["mlp.down"] = (self.down, 0)
+            if self.arr.gated_residual:
+                m["rg2"] = (self.up_gate, self.ff)
+                m["rg2.b"] = (self.rg2_b, 0)
+        return m
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        out = dict(self.mixer.cache_layout(block_size, dtype))
+        if self.shift is not None:
+            out["shift"] = ("slot", (self.width,), torch.float32)
+        return out
+
+    def forward(self, x, batch: ForwardBatch, cache: dict, dtype) -> None:
+        """x: fp32 residual rows [T, width], updated in place."""
+        if self.shift is not None:
+            xs, xa = ops.token_shift(
+                x, self.shift, cache["shift"], batch.cu_seqlens,
+                batch.seq_lens, batch.state_slots, batch.token_seq, dtype)
+        else:
+            xs = xa = x.to(dtype)
+        y = self.mixer(xs, batch, cache)
+        g = linear(xa, self.rg1) if self.rg1 is not None else None
+        xa = ops.gated_norm_residual(x, y, g, self.rg1_b, self.norm1, self.eps,
+                                     dtype if self.ff else None)
+        if self.ff:
+            ug = linear(xa, self.up_gate)
+            h = ops.gelu_tanh(ug[:, :self.ff])
+            y = linear(h, self.down)
+            g = ug[:, self.ff:] if self.arr.gated_residual else None
+            ops.gated_norm_residual(x, y, g, self.rg2_b, self.norm2, self.eps, None)
+
+
+class HybridForCausalLM(nn.Module):
+    supports_float32 = True
+    has_sequence_state = True  # engine: state slots, no prefix reuse
+
+    def __init__(self, cfg: HybridModelConfig, dtype=torch.bfloat16):
+        super().__init__()
+        if get_tp_world_size() != 1:
+            raise NotImplementedError(
+                f"{cfg.architecture}: tensor parallelism is not implemented")
+        self.cfg, self.dtype = cfg, dtype
+        arr = ARRANGEMENTS[cfg.architecture]
+        W = cfg.hidden_size
+        self.embed = _param(cfg.vocab_size, W, dtype=dtype)
+        self.layers = nn.ModuleList(
+            HybridBlock(W, spec, cfg.rms_norm_eps, dtype, arr)
+            for spec in cfg.layers)
+        self.final_norm = _param(W, dtype=torch.float32)
+        self.head = _param(cfg.vocab_size, W, dtype=dtype)
+        self._wmap = {"embed": (self.embed, 0), "head": (self.head, 0),
+                      "final.norm": (self.final_norm, 0)}
+        for i, layer in enumerate(self.layers):
+            for k, v in layer.weight_map().items():
+                self._wmap[f"l{i}.{k}"] = v
+        self._loaded: set = set()
+        self.residual_tap = None  # tests/tools: called with (layer, x)
+
+    # ------------------------------------------------------------ cache
+    def cache_layout(self, block_size: int) -> list:
+        return [layer.cache_layout(block_size, self.dtype) for layer in self.layers]
+
+    def kv_block_bytes(self, block_size: int) -> int:
+        total = 0
+        for layout in self.cache_layout(block_size):
+            for kind, shape, dt in layout.values():
+                if kind == "paged":
+                    total += int(torch.tensor(shape).prod()) * dt.itemsize
+        return max(total, 1)
+
+    def state_slot_bytes(self) -> int:
+        total = 0
+        for layout in self.cache_layout(16):
+            for kind, shape, dt in layout.values():
+                if kind == "slot":
+                    total += int(torch.tensor(shape).prod()) * dt.itemsize
+        return total
+
+    def allocate_cache(self, num_blocks: int, block_size: int, num_slots: int,
+                       device) -> list:
+        caches = []
+        for layout in self.cache_layout(block_size):
+            c = {}
+            for name, (kind, shape, dt) in layout.items():
+                lead = num_blocks if kind == "paged" else num_slots
+                c[name] = torch.zeros((lead, *shape), dtype=dt, device=device)
+            caches.append(c)
+        return caches
+
+    # ------------------------------------------------------------ forward
+    def forward(self, batch: ForwardBatch, caches: list) -> torch.Tensor:
+        """fp32 logits for batch.logits_indices rows (all rows if None)."""
+        x = self.embed[batch.input_ids].float()
+        for i, layer in enumerate(self.layers):
+            layer(x, batch, caches[i], self.dtype)
+            if self.residual_tap is not None:
+                self.residual_tap(i, x)
+        if batch.logits_indices is not None:
+            x = x[batch.logits_indices]
+        xn = ops.rms_norm_f32(x, self.final_norm, self.cfg.rms_norm_eps, self.dtype)
+        return linear(xn, self.head).float() * self.cfg.logit_scale
+
+    # ------------------------------------------------------------ weights
+    def load_hf_state_dict(self, tensors: dict) -> None:
+        """Tensors by their checkpoint names ('embed', 'l<i>.mix.q', ...);
+        fused parameters are filled span by span, in any order."""
+        for name, w in tensors.items():
+            if name not in self._wmap:
+                raise KeyError(f"unexpected tensor {name!r}")
+            p, row = self._wmap[name]
+            span = p.data[row:row + w.shape[0]] if w.dim() else p.data
+            if span.shape != w.shape:
+                raise ValueError(f"{name}: shape {tuple(w.shape)} does not fit "
+                                 f"{tuple(span.shape)}")
+            span.copy_(w.to(p.dtype))
+            self._loaded.add(name)
+        if len(self._loaded) == len(self._wmap):
+            self.finish_loading()
+
+    def finish_loading(self) -> None:
+        for layer in self.layers:
+            if hasattr(layer.mixer, "finish_loading"):
+                layer.mixer.finish_loading()
+
+    def missing_tensors(self) -> list:
+        return sorted(set(self._wmap) - self._loaded)
+
+    @torch.no_grad()
+    def random_init(self, seed: int = 0) -> None:
+        """Seeded random weights with activations of order one at every
+        block (benchmarks and tests; checkpoints load by name instead)."""
+        dev = self.embed.device
+        self._loaded.clear()
+        for name, (p, row) in self._wmap.items():
+            s = (seed * 1000003 + zlib.crc32(name.encode())) % (2 ** 63 - 1)
+            g = torch.Generator(device=dev).manual_seed(s)
+            leaf = name.split(".", 1)[1] if name.startswith("l") and "." in name else name
+            # rows of this tensor inside its (possibly fused) parameter
+            shape = list(p.shape)
+            if p.dim() == 2:
+                nxt = sorted(r for q, r in self._wmap.values() if q is p and r > row)
+                shape[0] = (nxt[0] if nxt else p.shape[0]) - row
+
+            def rn(std):
+                return torch.randn(shape, generator=g, device=dev,
+                                   dtype=torch.float32) * std
+
+            if leaf.endswith("norm") or leaf in ("norm1", "norm2"):
+                w = 1.0 + rn(0.1)
+            elif leaf == "shift":
+                w = torch.rand(shape, generator=g, device=dev)
+            elif leaf == "mix.A_log":
+                w = torch.log(1.0 + 7.0 * torch.rand(shape, generator=g, device=dev))
+            elif leaf == "mix.dt.b":
+                w = rn(0.5) - 3.0
+            elif leaf.endswith(".b") or leaf == "mix.D":
+                w = rn(0.3)
+            elif leaf == "embed":
+                w = rn(1.0)
+            else:
+                w = rn(shape[-1] ** -0.5)
+            self.load_hf_state_dict({name: w})

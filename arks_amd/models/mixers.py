@@ -1,0 +1,205 @@
+"""Sequence mixers for layer-list decoders, each with its constants as
+constructor parameters so that more than one design can use it:
+
+- SinkRotaryAttention: grouped-query softmax attention over the paged KV
+  cache with optional per-head q/k RMS norm, partial rotary (interleaved or
+  half-split pairs), a value-less sink key of score 0 in every softmax, and
+  values that are stored turned by their own position and turned back at
+  the query's position after the weighted sum.
+- LightningMixer: linear attention with one scalar decay per head and a
+  [dim x vdim] fp32 state per head and sequence, gated RMS-normed output.
+- Mamba1Mixer: short causal depthwise convolution + selective scan with an
+  [inner x state] fp32 state per sequence.
+
+Every mixer maps the (already token-shifted) rows [T, width] of one engine
+step to [T, width]; rows of several sequences are packed, prompt portions
+beside single decoded tokens, and ForwardBatch says where each sequence's
+rows, pages and state slot are. Projections run as library GEMMs in the
+model's dtype; everything that enters a softmax, a norm or a recurrence is
+fp32 inside the kernels (arks_amd/ops/csrc/seq_*.hip).
+
+Per-layer cache: each mixer names the tensors it needs in cache_layout():
+"paged" ones get a leading [num_blocks] axis and are addressed through the
+block tables, "slot" ones a leading [num_slots] axis addressed by
+ForwardBatch.state_slots.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .. import ops
+from ..engine.forward_batch import ForwardBatch
+
+
+def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x @ w^T as a library GEMM (the decode-shaped bf16 cases go to the
+    split-K kernel when the main extension is built)."""
+    if x.dtype == torch.bfloat16:
+        return ops.linear_bf16(x, w)
+    return F.linear(x, w)
+
+
+def _param(*shape, dtype):
+    return nn.Parameter(torch.zeros(*shape, dtype=dtype), requires_grad=False)
+
+
+def rotary_inv_freq(base: float, ndims: int) -> torch.Tensor:
+    """f_i = base^(-2i/ndims), i < ndims/2, rounded once from float64."""
+    i = torch.arange(ndims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64),
+                     -2.0 * i / ndims).float()
+
+
+class SinkRotaryAttention(nn.Module):
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, scale: float, rot_base: float, rot_dims: int,
+                 eps: float, dtype, qk_norm: bool = True, sink: bool = True,
+                 rotate_values: bool = True, interleaved: bool = True):
+        super().__init__()
+        assert heads % kv_heads == 0 and rot_dims % 2 == 0 and rot_dims <= dim
+        assert not rotate_values or vdim % 2 == 0
+        self.H, self.G, self.D, self.V = heads, kv_heads, dim, vdim
+        self.scale, self.eps = float(scale), eps
+        self.sink, self.interleaved = sink, interleaved
+        self.qkv = _param(heads * dim + kv_heads * (dim + vdim), width, dtype=dtype)
+        self.o = _param(width, heads * vdim, dtype=dtype)
+        self.q_norm = _param(dim, dtype=torch.float32) if qk_norm else None
+        self.k_norm = _param(dim, dtype=torch.float32) if qk_norm else None
+        self.register_buffer("inv_freq_qk", rotary_inv_freq(rot_base, rot_dims),
+                             persistent=False)
+        self.register_buffer(
+            "inv_freq_v",
+            rotary_inv_freq(rot_base, vdim) if rotate_values else None,
+            persistent=False)
+
+    def weight_map(self) -> dict:
+        H, G, D, V = self.H, self.G, self.D, self.V
+        m = {"q": (self.qkv, 0), "k": (self.qkv, H * D),
+             "v": (self.qkv, H * D + G * D), "o": (self.o, 0)}
+        if self.q_norm is not None:
+            m["q.norm"] = (self.q_norm, 0)
+            m["k.norm"] = (self.k_norm, 0)
+        return m
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        return {"k": ("paged", (self.G, block_size, self.D), dtype),
+                "v": ("paged", (self.G, block_size, self.V), dtype)}
+
+    def forward(self, xs, batch: ForwardBatch, cache: dict) -> torch.Tensor:
+        T = xs.shape[0]
+        H, G, D, V = self.H, self.G, self.D, self.V
+        qkv = linear(xs, self.qkv)
+        q = qkv[:, :H * D].unflatten(-1, (H, D))
+        k = qkv[:, H * D:(H + G) * D].unflatten(-1, (G, D))
+        v = qkv[:, (H + G) * D:].unflatten(-1, (G, V))
+        q = ops.qk_norm_rope_cache(
+            q, k, v, self.q_norm, self.k_norm, self.eps, batch.positions,
+            self.inv_freq_qk, self.inv_freq_v, cache["k"], cache["v"],
+            batch.slot_mapping, self.interleaved)
+        out = ops.attention_sink_paged(
+            q, cache["k"], cache["v"], batch.block_tables, batch.seq_lens,
+            batch.cu_seqlens, batch.token_seq, self.scale, self.sink,
+            self.inv_freq_v, self.interleaved, batch.max_q_len)
+        return linear(out.view(T, H * V), self.o)
+
+
+class LightningMixer(nn.Module):
+    def __init__(self, width: int, heads: int, dim: int, vdim: int,
+                 decay, eps: float, dtype):
+        super().__init__()
+        assert len(decay) == heads
+        self.H, self.D, self.V, self.eps = heads, dim, vdim, eps
+        self.qkvg = _param(2 * heads * dim + 2 * heads * vdim, width, dtype=dtype)
+        self.o = _param(width, heads * vdim, dtype=dtype)
+        self.norm = _param(heads * vdim, dtype=torch.float32)
+        self.register_buffer("decay", torch.tensor(
+            [float(d) for d in decay], dtype=torch.float64).float(),
+            persistent=False)
+
+    def weight_map(self) -> dict:
+        HD, HV = self.H * self.D, self.H * self.V
+        return {"q": (self.qkvg, 0), "k": (self.qkvg, HD),
+                "v": (self.qkvg, 2 * HD), "g": (self.qkvg, 2 * HD + HV),
+                "o": (self.o, 0), "norm": (self.norm, 0)}
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        return {"S": ("slot", (self.H, self.D, self.V), torch.float32)}
+
+    def forward(self, xs, batch: ForwardBatch, cache: dict) -> torch.Tensor:
+        T = xs.shape[0]
+        H, D, V = self.H, self.D, self.V
+        p = linear(xs, self.qkvg)
+        q = p[:, :H * D].unflatten(-1, (H, D))
+        k = p[:, H * D:2 * H * D].unflatten(-1, (H, D))
+        v = p[:, 2 * H * D:2 * H * D + H * V].unflatten(-1, (H, V))
+        g = p[:, 2 * H * D + H * V:]
+        o = ops.lightning_scan(q, k, v, self.decay, cache["S"],
+                               batch.cu_seqlens, batch.seq_lens,
+                               batch.state_slots, batch.max_q_len)
+        y = ops.gated_rmsnorm(o.view(T, H * V), self.norm, g, self.eps, xs.dtype)
+        return linear(y, self.o)
+
+
+class Mamba1Mixer(nn.Module):
+    def __init__(self, width: int, inner: int, state: int, dt_rank: int,
+                 conv: int, dtype):
+        super().__init__()
+        self.C, self.N, self.R, self.taps = inner, state, dt_rank, conv
+        self.w_in = _param(2 * inner, width, dtype=dtype)
+        self.w_x = _param(dt_rank + 2 * state, inner, dtype=dtype)
+        self.o = _param(width, inner, dtype=dtype)
+        f32 = torch.float32
+        self.conv_w = _param(inner, conv, dtype=f32)
+        self.conv_b = _param(inner, dtype=f32)
+        self.dt_w = _param(inner, dt_rank, dtype=f32)
+        self.dt_b = _param(inner, dtype=f32)
+        self.A_log = _param(inner, state, dtype=f32)
+        self.D = _param(inner, dtype=f32)
+        self.register_buffer("A", torch.zeros(inner, state, dtype=f32),
+                             persistent=False)
+
+    def weight_map(self) -> dict:
+        return {"in": (self.w_in, 0), "x": (self.w_x, 0), "o": (self.o, 0),
+                "conv": (self.conv_w, 0), "conv.b": (self.conv_b, 0),
+                "dt": (self.dt_w, 0), "dt.b": (self.dt_b, 0),
+                "A_log": (self.A_log, 0), "D": (self.D, 0)}
+
+    def finish_loading(self) -> None:
+        self.A.copy_(-torch.exp(self.A_log.data.float()))
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        out = {"ssm": ("slot", (self.C, self.N), torch.float32)}
+        if self.taps > 1:
+            out["conv"] = ("slot", (self.taps - 1, self.C), torch.float32)
+        return out
+
+    def forward(self, xs, batch: ForwardBatch, cache: dict) -> torch.Tensor:
+        C = self.C
+        xz = linear(xs, self.w_in)
+        u = ops.causal_conv_silu(
+            xz[:, :C], self.conv_w, self.conv_b, cache.get("conv"),
+            batch.cu_seqlens, batch.seq_lens, batch.state_slots,
+            batch.token_seq)
+        dbc = linear(u, self.w_x)
+        y = ops.selective_scan(
+            u, dbc, xz[:, C:], self.dt_w, self.dt_b, self.A, self.D,
+            cache["ssm"], batch.cu_seqlens, batch.seq_lens, batch.state_slots,
+            batch.max_q_len)
+        return linear(y, self.o)
+
+
+def build_mixer(kind: str, m: dict, width: int, eps: float, dtype) -> nn.Module:
+    if kind == "attention":
+        return SinkRotaryAttention(
+            width, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"],
+            m["rot"]["base"], m["rot"]["dims"], eps, dtype)
+    if kind == "lightning":
+        return LightningMixer(width, m["heads"], m["dim"], m["vdim"],
+                              m["decay"], eps, dtype)
+    if kind == "mamba1":
+        return Mamba1Mixer(width, m["inner"], m["state"], m["dt_rank"],
+                           m["conv"], dtype)
+    raise ValueError(f"unknown mixer type {kind!r}")

@@ -25,9 +25,9 @@ def _load_extension():
     if _C is not None or _C_ERR is not None:
         return _C
     try:
-        from . import _load  # noqa: F401  (imports the built .so in-tree)
+        from . import _load
 
-        _C = _load.C
+        _C = _load.load("arks_amd_C")  # the built .so in-tree
     except Exception as e:  # pragma: no cover - exercised only when unbuilt
         _C_ERR = f"{type(e).__name__}: {e}"
     return _C
@@ -539,3 +539,173 @@ def greedy_sample(logits):
         _native().greedy_sample(out, logits)
         return out
     return ref.greedy_sample(logits)
+
+
+# ----------------------------------------------------------------------
+# Sequence-state ops (arks_amd_seq_C): the kernels of the layer-list
+# decoders — token shift, gated output norm into an fp32 residual, sink
+# attention with rotated values, lightning linear attention, mamba1 conv
+# and selective scan. Same dispatch rule as above: CUDA tensors run the HIP
+# extension or fail loudly, CPU tensors run ops/ref.py.
+# ----------------------------------------------------------------------
+_S = None
+_S_ERR: str | None = None
+
+
+def _native_seq():
+    global _S, _S_ERR
+    if _S is None and _S_ERR is None:
+        try:
+            from . import _load
+
+            _S = _load.load("arks_amd_seq_C")
+        except Exception as e:
+            _S_ERR = f"{type(e).__name__}: {e}"
+    if _S is None:
+        raise RuntimeError(
+            "arks_amd sequence-state HIP extension (arks_amd_seq_C) is not "
+            "built but a GPU op was requested. Build it with `python -m "
+            f"arks_amd.ops.build arks_amd_seq_C` (import error: {_S_ERR})"
+        )
+    return _S
+
+
+def seq_native_available() -> bool:
+    try:
+        _native_seq()
+        return True
+    except RuntimeError:
+        return False
+
+
+def ensure_built(name: str) -> None:
+    """Compile one in-tree extension if its library is not there yet (a
+    fresh checkout on a GPU box); a no-op once built."""
+    global _S_ERR, _C_ERR
+    from .build import build, built_so_path
+
+    if built_so_path(name) is None:
+        build(name=name)
+        _S_ERR = _C_ERR = None
+
+
+def token_shift(x, shift_w, prev_state, cu_seqlens, seq_lens, state_slots,
+                token_seq, out_dtype):
+    """(xs, xa): the shifted mixer input and the plain row, both cast to
+    out_dtype; prev_state takes each sequence's last row."""
+    if x.is_cuda:
+        xs = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        xa = xs if out_dtype == torch.float32 else torch.empty_like(xs)
+        _native_seq().token_shift(xs, xa, x, shift_w, prev_state, cu_seqlens,
+                                  seq_lens, state_slots, token_seq)
+        return xs, (x if out_dtype == torch.float32 else xa)
+    return ref.token_shift(x, shift_w, prev_state, cu_seqlens, seq_lens,
+                           state_slots, out_dtype)
+
+
+def gated_norm_residual(x, y, gate, gate_bias, weight, eps, out_dtype=None):
+    """x (fp32, in place) += rmsnorm(y * sigmoid(gate + bias)) * weight.
+    Returns the new x cast to out_dtype when one is asked for."""
+    if x.is_cuda:
+        if out_dtype == torch.float32:
+            out_dtype = None  # x itself is the fp32 copy
+            ret_x = True
+        else:
+            ret_x = False
+        xa = (torch.empty(x.shape, dtype=out_dtype, device=x.device)
+              if out_dtype is not None else None)
+        _native_seq().gated_norm_residual(x, xa, y, gate, gate_bias, weight, eps)
+        return x if ret_x else xa
+    return ref.gated_norm_residual(x, y, gate, gate_bias, weight, eps, out_dtype)
+
+
+def rms_norm_f32(x, weight, eps, out_dtype):
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _native_seq().rms_norm_f32(out, x, weight, eps)
+        return out
+    return ref.rms_norm_f32(x, weight, eps, out_dtype)
+
+
+def qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
+                       inv_freq_qk, inv_freq_v, k_cache, v_cache,
+                       slot_mapping, interleaved=True):
+    if q.is_cuda:
+        T, H, D = q.shape
+        qo = torch.empty((T, H, D), dtype=q.dtype, device=q.device)
+        _native_seq().qk_norm_rope_cache(
+            qo, q, k, v, q_norm_w, k_norm_w, eps, positions, inv_freq_qk,
+            inv_freq_v, k_cache, v_cache, slot_mapping, interleaved)
+        return qo
+    return ref.qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
+                                  inv_freq_qk, inv_freq_v, k_cache, v_cache,
+                                  slot_mapping, interleaved)
+
+
+def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
+                         cu_seqlens, token_seq, scale, sink=True,
+                         inv_freq_v=None, interleaved=True, max_q_len=0):
+    if q.is_cuda:
+        T, H, _ = q.shape
+        V = v_cache.shape[3]
+        out = torch.empty((T, H, V), dtype=q.dtype, device=q.device)
+        _native_seq().attention_sink_paged(
+            out, q, k_cache, v_cache, block_tables, seq_lens, cu_seqlens,
+            token_seq, scale, sink, inv_freq_v, interleaved, max_q_len)
+        return out
+    return ref.attention_sink_paged(q, k_cache, v_cache, block_tables,
+                                    seq_lens, cu_seqlens, scale, sink,
+                                    inv_freq_v, interleaved)
+
+
+def lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
+                   max_q_len=0):
+    if q.is_cuda:
+        T, H, _ = q.shape
+        V = v.shape[2]
+        out = torch.empty((T, H, V), dtype=torch.float32, device=q.device)
+        _native_seq().lightning_scan(out, q, k, v, decay, state, cu_seqlens,
+                                     seq_lens, state_slots, max_q_len)
+        return out
+    return ref.lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens,
+                              state_slots)
+
+
+def gated_rmsnorm(o, weight, gate, eps, out_dtype):
+    if o.is_cuda:
+        out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
+        _native_seq().gated_rmsnorm(out, o, weight, gate, eps)
+        return out
+    return ref.gated_rmsnorm(o, weight, gate, eps, out_dtype)
+
+
+def causal_conv_silu(x, weight, bias, state, cu_seqlens, seq_lens,
+                     state_slots, token_seq):
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _native_seq().causal_conv_silu(out, x, weight, bias, state, cu_seqlens,
+                                       seq_lens, state_slots, token_seq)
+        return out
+    return ref.causal_conv_silu(x, weight, bias, state, cu_seqlens, seq_lens,
+                                state_slots)
+
+
+def selective_scan(u, dbc, z, dt_w, dt_b, A, Dp, state, cu_seqlens, seq_lens,
+                   state_slots, max_q_len=0):
+    if u.is_cuda:
+        out = torch.empty(u.shape, dtype=u.dtype, device=u.device)
+        _native_seq().selective_scan(out, u, dbc, z, dt_w, dt_b, A, Dp, state,
+                                     cu_seqlens, seq_lens, state_slots,
+                                     max_q_len)
+        return out
+    return ref.selective_scan(u, dbc, z, dt_w, dt_b, A, Dp, state, cu_seqlens,
+                              seq_lens, state_slots)
+
+
+def gelu_tanh(x):
+    """tanh-form GELU; x may be a column slice of a wider GEMM output."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _native_seq().gelu_tanh(out, x)
+        return out
+    return ref.gelu_tanh(x)

@@ -1,4 +1,4 @@
-"""Imports the in-tree built HIP extension (arks_amd/ops/_build/arks_amd_C.so).
+"""Imports the in-tree built HIP extensions (arks_amd/ops/_build/<name>/<name>.so).
 
 Raises ImportError if the extension has not been built — callers on a GPU box
 must fail loudly rather than fall back to eager PyTorch.
@@ -12,13 +12,16 @@ import torch  # noqa: F401  (the extension links against libtorch)
 
 from .build import built_so_path
 
-_so = built_so_path()
-if _so is None:
-    raise ImportError(
-        "arks_amd_C.so not found in arks_amd/ops/_build — run "
-        "`python -m arks_amd.ops.build`"
-    )
 
-_spec = importlib.util.spec_from_file_location("arks_amd_C", _so)
-C = importlib.util.module_from_spec(_spec)
-_spec.loader.exec_module(C)
+
+def load(name: str):
+    so = built_so_path(name)
+    if so is None:
+        raise ImportError(
+            f"{name}.so not found in arks_amd/ops/_build/{name} — run "
+            f"`python -m arks_amd.ops.build {name}`"
+        )
+    spec = importlib.util.spec_from_file_location(name, so)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod

@@ -34,31 +34,58 @@ SOURCES = [
 ]
 
 
-def built_so_path() -> str | None:
-    matches = glob.glob(os.path.join(BUILD_DIR, f"{EXT_NAME}*.so"))
+# The sequence-state kernels (layer-list decoders) are a library of their
+# own: a checkout that only serves such a model compiles these few files.
+SEQ_EXT_NAME = "arks_amd_seq_C"
+SEQ_SOURCES = [
+    os.path.join(CSRC, "seq_bindings.cpp"),
+    os.path.join(CSRC, "seq_elementwise.hip"),
+    os.path.join(CSRC, "seq_attention.hip"),
+    os.path.join(CSRC, "seq_lightning.hip"),
+    os.path.join(CSRC, "seq_mamba.hip"),
+]
+
+EXTENSIONS = {EXT_NAME: SOURCES, SEQ_EXT_NAME: SEQ_SOURCES}
+
+# hipcc only: ordinary float code must not be turned into packed-fp32 ops
+HIPCC_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def built_so_path(name: str = EXT_NAME) -> str | None:
+    matches = glob.glob(os.path.join(BUILD_DIR, name, f"{name}*.so"))
     return matches[0] if matches else None
 
 
-def build(verbose: bool = False):
+def build(verbose: bool = False, name: str | None = None):
+    """Compile one extension (or all of them) in-tree; returns the path of
+    the last library built."""
     os.environ.setdefault("PYTORCH_ROCM_ARCH", "gfx950")
-    os.makedirs(BUILD_DIR, exist_ok=True)
     from torch.utils import cpp_extension
 
-    cpp_extension.load(
-        name=EXT_NAME,
-        sources=SOURCES,
-        extra_cflags=["-O3", "-std=c++17"],
-        extra_cuda_cflags=["-O3", "-std=c++17", "--offload-arch=gfx950"],
-        build_directory=BUILD_DIR,
-        verbose=verbose,
-        is_python_module=False,  # we import the .so ourselves (_load.py)
-        keep_intermediates=True,
-    )
-    so = built_so_path()
-    assert so is not None, "build produced no .so"
+    so = None
+    for ext, sources in EXTENSIONS.items():
+        if name is not None and ext != name:
+            continue
+        out_dir = os.path.join(BUILD_DIR, ext)
+        os.makedirs(out_dir, exist_ok=True)
+        cpp_extension.load(
+            name=ext,
+            sources=sources,
+            extra_cflags=["-O3", "-std=c++17"],
+            extra_cuda_cflags=HIPCC_FLAGS,
+            build_directory=out_dir,
+            verbose=verbose,
+            is_python_module=False,  # we import the .so ourselves (_load.py)
+            keep_intermediates=True,
+        )
+        so = built_so_path(ext)
+        assert so is not None, f"build of {ext} produced no .so"
+    assert so is not None, f"unknown extension {name!r}"
     return so
 
 
 if __name__ == "__main__":
-    so = build(verbose="-v" in sys.argv)
-    print(f"built: {so}")
+    names = [a for a in sys.argv[1:] if not a.startswith("-")]
+    for n in names or [None]:
+        print(f"built: {build(verbose='-v' in sys.argv, name=n)}")

@@ -1,0 +1,402 @@
+// Python bindings of the sequence-state kernels (arks_amd_seq_C). Shapes,
+// dtypes and strides are validated here; the kernels are in seq_*.hip.
+#include <torch/extension.h>
+
+#include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime.h>
+
+extern "C" {
+void arks_seq_token_shift(void* xs, void* xa, const void* x, const void* w,
+                          void* state, const void* cu, const void* seq_lens,
+                          const void* slots, const void* token_seq, int T,
+                          int W, int act_f32, hipStream_t stream);
+void arks_seq_gated_norm_residual(void* x, void* xa, const void* y,
+                                  const void* g, int64_t ldg, const void* gb,
+                                  const void* w, float eps, int T, int W,
+                                  int act_f32, hipStream_t stream);
+void arks_seq_rms_norm_f32(void* out, const void* x, const void* w,
+                           const void* gate, int64_t ldg, float eps, int T,
+                           int W, int act_f32, hipStream_t stream);
+void arks_seq_gelu_tanh(void* out, const void* x, int64_t ldx, int64_t rows,
+                        int n, int act_f32, hipStream_t stream);
+void arks_seq_qk_norm_rope_cache(
+    void* qo, const void* q, const void* k, const void* v, int64_t ldq,
+    int64_t ldk, int64_t ldv, const void* qw, const void* kw, float eps,
+    const void* positions, const void* freq_qk, int n_rot, const void* freq_v,
+    int n_vrot, void* k_cache, void* v_cache, const void* slot_mapping, int T,
+    int H, int G, int D, int V, int block_size, int interleaved, int act_f32,
+    hipStream_t stream);
+int arks_seq_attn_sink_generic(
+    void* out, const void* q, const void* k_cache, const void* v_cache,
+    const void* block_tables, const void* seq_lens, const void* cu,
+    const void* token_seq, float scale, int sink, const void* freq_v,
+    int interleaved, int T, int H, int G, int D, int V, int block_size,
+    int max_blocks, int act_f32, hipStream_t stream);
+int arks_seq_lightning_scan(void* out, const void* q, const void* k,
+                            const void* v, int64_t ldq, int64_t ldk,
+                            int64_t ldv, const void* decay, void* state,
+                            const void* cu, const void* seq_lens,
+                            const void* slots, int S, int H, int D, int V,
+                            int act_f32, hipStream_t stream);
+int arks_seq_causal_conv_silu(void* out, const void* x, int64_t ldx,
+                              const void* w, const void* bias, void* state,
+                              const void* cu, const void* seq_lens,
+                              const void* slots, const void* token_seq, int T,
+                              int S, int C, int taps, int act_f32,
+                              hipStream_t stream);
+int arks_seq_selective_scan(void* out, const void* u, const void* dbc,
+                            int64_t ldd, const void* z, int64_t ldz,
+                            const void* dt_w, const void* dt_b, const void* A,
+                            const void* Dp, void* state, const void* cu,
+                            const void* seq_lens, const void* slots, int S,
+                            int C, int N, int R, int act_f32,
+                            hipStream_t stream);
+}
+
+namespace {
+
+using torch::Tensor;
+using OptTensor = c10::optional<Tensor>;
+
+hipStream_t current_stream() {
+  return c10::hip::getCurrentHIPStream().stream();
+}
+
+int act_flag(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda(), name, " must be on the GPU");
+  TORCH_CHECK(t.scalar_type() == torch::kBFloat16 ||
+                  t.scalar_type() == torch::kFloat32,
+              name, " must be bfloat16 or float32");
+  return t.scalar_type() == torch::kFloat32 ? 1 : 0;
+}
+
+void check_f32(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kFloat32 &&
+                  t.is_contiguous(),
+              name, " must be a contiguous float32 GPU tensor");
+}
+
+void check_i32(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kInt32 &&
+                  t.is_contiguous(),
+              name, " must be a contiguous int32 GPU tensor");
+}
+
+void check_i64(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == torch::kInt64 &&
+                  t.is_contiguous(),
+              name, " must be a contiguous int64 GPU tensor");
+}
+
+// rows x cols view whose last dim is dense; returns the row stride
+int64_t row_stride(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.dim() == 2 && t.stride(1) == 1, name,
+              " must be 2-D with a dense last dim");
+  return t.stride(0);
+}
+
+// [T, heads, dim] view of a wider row: heads dense
+int64_t head_row_stride(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.dim() == 3 && t.stride(2) == 1 && t.stride(1) == t.size(2),
+              name, " must be [T, heads, dim] with dense heads");
+  return t.stride(0);
+}
+
+struct SeqMeta {
+  int S;
+};
+
+SeqMeta check_meta(const Tensor& cu, const Tensor& seq_lens,
+                   const Tensor* slots, const Tensor* token_seq, int64_t T) {
+  check_i32(cu, "cu_seqlens");
+  check_i32(seq_lens, "seq_lens");
+  const int64_t S = seq_lens.numel();
+  TORCH_CHECK(cu.numel() == S + 1, "cu_seqlens must have num_seqs + 1 entries");
+  if (slots) {
+    check_i32(*slots, "state_slots");
+    TORCH_CHECK(slots->numel() == S, "state_slots must have num_seqs entries");
+  }
+  if (token_seq) {
+    check_i32(*token_seq, "token_seq");
+    TORCH_CHECK(token_seq->numel() == T, "token_seq must have one entry per row");
+  }
+  return {(int)S};
+}
+
+void token_shift(Tensor xs, Tensor xa, Tensor x, Tensor w, Tensor state,
+                 Tensor cu, Tensor seq_lens, Tensor slots, Tensor token_seq) {
+  check_f32(x, "x");
+  check_f32(w, "shift weight");
+  check_f32(state, "shift state");
+  const int T = x.size(0), W = x.size(1);
+  const int f32 = act_flag(xs, "xs");
+  TORCH_CHECK(xs.is_contiguous() && xs.sizes() == x.sizes());
+  TORCH_CHECK(w.numel() == W && state.dim() == 2 && state.size(1) == W);
+  check_meta(cu, seq_lens, &slots, &token_seq, T);
+  void* xa_p = nullptr;
+  if (!f32) {
+    TORCH_CHECK(xa.scalar_type() == xs.scalar_type() && xa.is_contiguous() &&
+                xa.sizes() == x.sizes());
+    xa_p = xa.data_ptr();
+  }
+  arks_seq_token_shift(xs.data_ptr(), xa_p, x.data_ptr(), w.data_ptr(),
+                       state.data_ptr(), cu.data_ptr(), seq_lens.data_ptr(),
+                       slots.data_ptr(), token_seq.data_ptr(), T, W, f32,
+                       current_stream());
+}
+
+void gated_norm_residual(Tensor x, OptTensor xa, Tensor y, OptTensor gate,
+                         OptTensor gate_bias, Tensor w, double eps) {
+  check_f32(x, "x");
+  check_f32(w, "norm weight");
+  const int T = x.size(0), W = x.size(1);
+  const int f32 = act_flag(y, "y");
+  TORCH_CHECK(y.is_contiguous() && y.dim() == 2 && y.size(0) == T &&
+              y.size(1) == W, "y must be contiguous [T, W]");
+  TORCH_CHECK(w.numel() == W);
+  const void* g_p = nullptr;
+  const void* gb_p = nullptr;
+  int64_t ldg = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->scalar_type() == y.scalar_type() && gate->size(0) == T &&
+                gate->size(1) == W);
+    ldg = row_stride(*gate, "gate");
+    TORCH_CHECK(gate_bias.has_value());
+    check_f32(*gate_bias, "gate bias");
+    TORCH_CHECK(gate_bias->numel() == W);
+    g_p = gate->data_ptr();
+    gb_p = gate_bias->data_ptr();
+  }
+  void* xa_p = nullptr;
+  if (xa.has_value()) {
+    TORCH_CHECK(xa->scalar_type() == y.scalar_type() && xa->is_contiguous() &&
+                xa->sizes() == x.sizes());
+    xa_p = xa->data_ptr();
+  }
+  arks_seq_gated_norm_residual(x.data_ptr(), xa_p, y.data_ptr(), g_p, ldg, gb_p,
+                               w.data_ptr(), (float)eps, T, W, f32,
+                               current_stream());
+}
+
+void rms_norm_f32(Tensor out, Tensor x, Tensor w, double eps) {
+  check_f32(x, "x");
+  check_f32(w, "norm weight");
+  const int f32 = act_flag(out, "out");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes() && x.dim() == 2);
+  TORCH_CHECK(w.numel() == x.size(1));
+  arks_seq_rms_norm_f32(out.data_ptr(), x.data_ptr(), w.data_ptr(), nullptr, 0,
+                        (float)eps, x.size(0), x.size(1), f32, current_stream());
+}
+
+void gated_rmsnorm(Tensor out, Tensor o, Tensor w, Tensor gate, double eps) {
+  check_f32(o, "o");
+  check_f32(w, "norm weight");
+  const int f32 = act_flag(out, "out");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == o.sizes() && o.dim() == 2);
+  TORCH_CHECK(gate.scalar_type() == out.scalar_type() &&
+              gate.size(0) == o.size(0) && gate.size(1) == o.size(1));
+  TORCH_CHECK(w.numel() == o.size(1));
+  arks_seq_rms_norm_f32(out.data_ptr(), o.data_ptr(), w.data_ptr(),
+                        gate.data_ptr(), row_stride(gate, "gate"), (float)eps,
+                        o.size(0), o.size(1), f32, current_stream());
+}
+
+void gelu_tanh(Tensor out, Tensor x) {
+  const int f32 = act_flag(x, "x");
+  TORCH_CHECK(out.scalar_type() == x.scalar_type() && out.is_contiguous() &&
+              out.sizes() == x.sizes());
+  arks_seq_gelu_tanh(out.data_ptr(), x.data_ptr(), row_stride(x, "x"),
+                     x.size(0), x.size(1), f32, current_stream());
+}
+
+void qk_norm_rope_cache(Tensor qo, Tensor q, Tensor k, Tensor v, OptTensor qw,
+                        OptTensor kw, double eps, Tensor positions,
+                        Tensor freq_qk, OptTensor freq_v, Tensor k_cache,
+                        Tensor v_cache, Tensor slot_mapping, bool interleaved) {
+  const int f32 = act_flag(q, "q");
+  const int T = q.size(0), H = q.size(1), D = q.size(2);
+  const int G = k.size(1), V = v.size(2);
+  TORCH_CHECK(k.scalar_type() == q.scalar_type() &&
+              v.scalar_type() == q.scalar_type() &&
+              qo.scalar_type() == q.scalar_type() &&
+              k_cache.scalar_type() == q.scalar_type() &&
+              v_cache.scalar_type() == q.scalar_type(),
+              "q, k, v and the cache must share one dtype");
+  TORCH_CHECK(k.size(0) == T && v.size(0) == T && k.size(2) == D &&
+              v.size(1) == G);
+  TORCH_CHECK(qo.is_contiguous() && qo.sizes() == q.sizes());
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.dim() == 4 && v_cache.dim() == 4);
+  TORCH_CHECK(k_cache.size(1) == G && k_cache.size(3) == D &&
+              v_cache.size(1) == G && v_cache.size(3) == V &&
+              v_cache.size(2) == k_cache.size(2) &&
+              v_cache.size(0) == k_cache.size(0), "cache shape mismatch");
+  check_i64(positions, "positions");
+  check_i64(slot_mapping, "slot_mapping");
+  TORCH_CHECK(positions.numel() == T && slot_mapping.numel() == T);
+  check_f32(freq_qk, "inv_freq_qk");
+  const int n_rot = freq_qk.numel();
+  TORCH_CHECK(2 * n_rot <= D, "rotary dims exceed the head size");
+  const void* qw_p = nullptr;
+  const void* kw_p = nullptr;
+  if (qw.has_value()) {
+    check_f32(*qw, "q norm weight");
+    TORCH_CHECK(kw.has_value());
+    check_f32(*kw, "k norm weight");
+    TORCH_CHECK(qw->numel() == D && kw->numel() == D);
+    qw_p = qw->data_ptr();
+    kw_p = kw->data_ptr();
+  }
+  const void* fv_p = nullptr;
+  int n_vrot = 0;
+  if (freq_v.has_value()) {
+    check_f32(*freq_v, "inv_freq_v");
+    n_vrot = freq_v->numel();
+    TORCH_CHECK(2 * n_vrot == V, "value rotation covers all value dims");
+    fv_p = freq_v->data_ptr();
+  }
+  arks_seq_qk_norm_rope_cache(
+      qo.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+      head_row_stride(q, "q"), head_row_stride(k, "k"), head_row_stride(v, "v"),
+      qw_p, kw_p, (float)eps, positions.data_ptr(), freq_qk.data_ptr(), n_rot,
+      fv_p, n_vrot, k_cache.data_ptr(), v_cache.data_ptr(),
+      slot_mapping.data_ptr(), T, H, G, D, V, (int)k_cache.size(2),
+      interleaved ? 1 : 0, f32, current_stream());
+}
+
+void attention_sink_paged(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                          Tensor block_tables, Tensor seq_lens, Tensor cu,
+                          Tensor token_seq, double scale, bool sink,
+                          OptTensor freq_v, bool interleaved,
+                          int64_t max_q_len) {
+  const int f32 = act_flag(q, "q");
+  TORCH_CHECK(q.is_contiguous() && q.dim() == 3);
+  const int T = q.size(0), H = q.size(1), D = q.size(2);
+  TORCH_CHECK(k_cache.scalar_type() == q.scalar_type() &&
+              v_cache.scalar_type() == q.scalar_type() &&
+              out.scalar_type() == q.scalar_type());
+  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.size(3) == D);
+  const int G = k_cache.size(1), bs = k_cache.size(2), V = v_cache.size(3);
+  TORCH_CHECK(H % G == 0 && v_cache.size(1) == G && v_cache.size(2) == bs);
+  TORCH_CHECK(out.is_contiguous() && out.size(0) == T && out.size(1) == H &&
+              out.size(2) == V);
+  check_i32(block_tables, "block_tables");
+  TORCH_CHECK(block_tables.dim() == 2 &&
+              block_tables.size(0) == seq_lens.numel());
+  check_meta(cu, seq_lens, nullptr, &token_seq, T);
+  const void* fv_p = nullptr;
+  if (freq_v.has_value()) {
+    check_f32(*freq_v, "inv_freq_v");
+    TORCH_CHECK(2 * freq_v->numel() == V);
+    fv_p = freq_v->data_ptr();
+  }
+  const int rc = arks_seq_attn_sink_generic(
+      out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+      block_tables.data_ptr(), seq_lens.data_ptr(), cu.data_ptr(),
+      token_seq.data_ptr(), (float)scale, sink ? 1 : 0, fv_p,
+      interleaved ? 1 : 0, T, H, G, D, V, bs, (int)block_tables.size(1), f32,
+      current_stream());
+  TORCH_CHECK(rc == 0, "attention head sizes beyond the kernel's limits (",
+              D, ", ", V, ")");
+}
+
+void lightning_scan(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
+                    Tensor state, Tensor cu, Tensor seq_lens, Tensor slots,
+                    int64_t max_q_len) {
+  const int f32 = act_flag(q, "q");
+  const int T = q.size(0), H = q.size(1), D = q.size(2), V = v.size(2);
+  TORCH_CHECK(k.scalar_type() == q.scalar_type() &&
+              v.scalar_type() == q.scalar_type());
+  TORCH_CHECK(k.size(0) == T && k.size(1) == H && k.size(2) == D &&
+              v.size(0) == T && v.size(1) == H);
+  check_f32(out, "out");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H && out.size(2) == V);
+  check_f32(decay, "decay");
+  TORCH_CHECK(decay.numel() == H);
+  check_f32(state, "state");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D &&
+              state.size(3) == V, "state must be [slots, H, D, V]");
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, nullptr, T);
+  const int rc = arks_seq_lightning_scan(
+      out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+      head_row_stride(q, "q"), head_row_stride(k, "k"), head_row_stride(v, "v"),
+      decay.data_ptr(), state.data_ptr(), cu.data_ptr(), seq_lens.data_ptr(),
+      slots.data_ptr(), m.S, H, D, V, f32, current_stream());
+  TORCH_CHECK(rc == 0, "lightning head size beyond the kernel's limit (", D, ")");
+}
+
+void causal_conv_silu(Tensor out, Tensor x, Tensor w, Tensor bias,
+                      OptTensor state, Tensor cu, Tensor seq_lens, Tensor slots,
+                      Tensor token_seq) {
+  const int f32 = act_flag(x, "x");
+  const int T = x.size(0), C = x.size(1);
+  TORCH_CHECK(out.scalar_type() == x.scalar_type() && out.is_contiguous() &&
+              out.sizes() == x.sizes());
+  check_f32(w, "conv weight");
+  check_f32(bias, "conv bias");
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C && bias.numel() == C);
+  const int taps = w.size(1);
+  void* st_p = nullptr;
+  if (taps > 1) {
+    TORCH_CHECK(state.has_value());
+    check_f32(*state, "conv state");
+    TORCH_CHECK(state->dim() == 3 && state->size(1) == taps - 1 &&
+                state->size(2) == C, "conv state must be [slots, taps-1, C]");
+    st_p = state->data_ptr();
+  }
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, &token_seq, T);
+  const int rc = arks_seq_causal_conv_silu(
+      out.data_ptr(), x.data_ptr(), row_stride(x, "x"), w.data_ptr(),
+      bias.data_ptr(), st_p, cu.data_ptr(), seq_lens.data_ptr(),
+      slots.data_ptr(), token_seq.data_ptr(), T, m.S, C, taps, f32,
+      current_stream());
+  TORCH_CHECK(rc == 0, "conv taps beyond the kernel's limit (", taps, ")");
+}
+
+void selective_scan(Tensor out, Tensor u, Tensor dbc, Tensor z, Tensor dt_w,
+                    Tensor dt_b, Tensor A, Tensor Dp, Tensor state, Tensor cu,
+                    Tensor seq_lens, Tensor slots, int64_t max_q_len) {
+  const int f32 = act_flag(u, "u");
+  const int T = u.size(0), C = u.size(1);
+  TORCH_CHECK(u.is_contiguous() && out.is_contiguous() &&
+              out.scalar_type() == u.scalar_type() && out.sizes() == u.sizes());
+  TORCH_CHECK(dbc.scalar_type() == u.scalar_type() &&
+              z.scalar_type() == u.scalar_type());
+  check_f32(dt_w, "dt weight");
+  check_f32(dt_b, "dt bias");
+  check_f32(A, "A");
+  check_f32(Dp, "D");
+  check_f32(state, "ssm state");
+  const int R = dt_w.size(1), N = A.size(1);
+  TORCH_CHECK(dt_w.size(0) == C && dt_b.numel() == C && A.size(0) == C &&
+              Dp.numel() == C);
+  TORCH_CHECK(dbc.size(0) == T && dbc.size(1) == R + 2 * N,
+              "dbc must be [T, dt_rank + 2 * state]");
+  TORCH_CHECK(z.size(0) == T && z.size(1) == C);
+  TORCH_CHECK(state.dim() == 3 && state.size(1) == C && state.size(2) == N,
+              "ssm state must be [slots, C, N]");
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, nullptr, T);
+  const int rc = arks_seq_selective_scan(
+      out.data_ptr(), u.data_ptr(), dbc.data_ptr(), row_stride(dbc, "dbc"),
+      z.data_ptr(), row_stride(z, "z"), dt_w.data_ptr(), dt_b.data_ptr(),
+      A.data_ptr(), Dp.data_ptr(), state.data_ptr(), cu.data_ptr(),
+      seq_lens.data_ptr(), slots.data_ptr(), m.S, C, N, R, f32,
+      current_stream());
+  TORCH_CHECK(rc == 0, "ssm state size beyond the kernel's limit (", N, ")");
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("token_shift", &token_shift);
+  m.def("gated_norm_residual", &gated_norm_residual);
+  m.def("rms_norm_f32", &rms_norm_f32);
+  m.def("gated_rmsnorm", &gated_rmsnorm);
+  m.def("gelu_tanh", &gelu_tanh);
+  m.def("qk_norm_rope_cache", &qk_norm_rope_cache);
+  m.def("attention_sink_paged", &attention_sink_paged);
+  m.def("lightning_scan", &lightning_scan);
+  m.def("causal_conv_silu", &causal_conv_silu);
+  m.def("selective_scan", &selective_scan);
+}

@@ -1,0 +1,234 @@
+// Row-wise kernels around the fp32 residual stream of the layer-list
+// decoders: token shift, gated output norm + residual add, final norm,
+// gated RMS norm, tanh-GELU, and the attention front end (per-head q/k RMS
+// norm, rotary, position-turned values, paged cache write).
+#include "seq_common.h"
+
+namespace arks {
+
+// xs[t] = x[t] + (x[t-1] - x[t]) * w, x[-1] = the sequence's stored last
+// row (or 0 at position 0). The block of a sequence's FIRST row is the only
+// reader of the stored row, and the one that replaces it with the last row
+// of this step — same thread, read before write, so no ordering between
+// blocks is needed.
+template <typename AT>
+__global__ __launch_bounds__(256) void token_shift_kernel(
+    AT* __restrict__ xs, AT* __restrict__ xa, const float* __restrict__ x,
+    const float* __restrict__ w, float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ seq_lens,
+    const int* __restrict__ slots, const int* __restrict__ token_seq, int W) {
+  const int t = blockIdx.x;
+  const SeqRow r = seq_row(t, token_seq, cu, seq_lens, slots);
+  const bool first = (t == r.first_row);
+  const bool has_state = r.start > 0 && r.slot >= 0;
+  const float* xr = x + (int64_t)t * W;
+  const float* xp = x + (int64_t)(t - 1) * W;
+  const float* xl = x + (int64_t)(r.first_row + r.rows - 1) * W;
+  float* st = state + (int64_t)(r.slot < 0 ? 0 : r.slot) * W;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    const float xv = xr[i];
+    const float prev = first ? (has_state ? st[i] : 0.f) : xp[i];
+    Act<AT>::st(xs + (int64_t)t * W + i, xv + (prev - xv) * w[i]);
+    if (xa) Act<AT>::st(xa + (int64_t)t * W + i, xv);
+    if (first && r.slot >= 0) st[i] = xl[i];
+  }
+}
+
+// x += rmsnorm(y * sigmoid(g + gb)) * w ; optional cast copy of the new x.
+template <typename AT>
+__global__ __launch_bounds__(256) void gated_norm_residual_kernel(
+    float* __restrict__ x, AT* __restrict__ xa, const AT* __restrict__ y,
+    const AT* __restrict__ g, int64_t ldg, const float* __restrict__ gb,
+    const float* __restrict__ w, float eps, int W) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const AT* yr = y + (int64_t)t * W;
+  const AT* gr = g ? g + (int64_t)t * ldg : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    float z = Act<AT>::ld(yr + i);
+    if (gr) z *= sigmoid_f(Act<AT>::ld(gr + i) + gb[i]);
+    ss += z * z;
+  }
+  ss = block_reduce_sum<256>(ss, scratch);
+  const float rstd = 1.f / sqrtf(ss / (float)W + eps);
+  float* xr = x + (int64_t)t * W;
+  for (int i = threadIdx.x; i < W; i += 256) {
+    float z = Act<AT>::ld(yr + i);
+    if (gr) z *= sigmoid_f(Act<AT>::ld(gr + i) + gb[i]);
+    const float nx = xr[i] + z * rstd * w[i];
+    xr[i] = nx;
+    if (xa) Act<AT>::st(xa + (int64_t)t * W + i, nx);
+  }
+}
+
+// out = rmsnorm(x) * w [* sigmoid(gate)], x fp32.
+template <typename AT>
+__global__ __launch_bounds__(256) void rms_norm_f32_kernel(
+    AT* __restrict__ out, const float* __restrict__ x,
+    const float* __restrict__ w, const AT* __restrict__ gate, int64_t ldg,
+    float eps, int W) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const float* xr = x + (int64_t)t * W;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < W; i += 256) ss += xr[i] * xr[i];
+  ss = block_reduce_sum<256>(ss, scratch);
+  const float rstd = 1.f / sqrtf(ss / (float)W + eps);
+  for (int i = threadIdx.x; i < W; i += 256) {
+    float v = xr[i] * rstd * w[i];
+    if (gate) v *= sigmoid_f(Act<AT>::ld(gate + (int64_t)t * ldg + i));
+    Act<AT>::st(out + (int64_t)t * W + i, v);
+  }
+}
+
+template <typename AT>
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(
+    AT* __restrict__ out, const AT* __restrict__ x, int64_t ldx, int64_t rows,
+    int n) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * n) return;
+  const int64_t r = idx / n;
+  const int c = (int)(idx - r * n);
+  const float z = Act<AT>::ld(x + r * ldx + c);
+  const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  Act<AT>::st(out + idx, 0.5f * z * (1.f + tanhf(u)));
+}
+
+// One wave per (row, head slot): slots [0,H) are query heads, [H,H+G) key
+// heads, [H+G,H+2G) value heads. q/k: RMS norm over the head (weight or
+// none) then rotary on the first 2*n_rot dims; v: turned by the row's
+// position over all its dims (n_vrot pairs; 0 = stored plain). Pairs are
+// (2i,2i+1) when interleaved, (i, i+n) otherwise. k and v go to their page.
+template <typename AT>
+__global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
+    AT* __restrict__ qo, const AT* __restrict__ q, const AT* __restrict__ k,
+    const AT* __restrict__ v, int64_t ldq, int64_t ldk, int64_t ldv,
+    const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+    const int64_t* __restrict__ positions, const float* __restrict__ freq_qk,
+    int n_rot, const float* __restrict__ freq_v, int n_vrot,
+    AT* __restrict__ k_cache, AT* __restrict__ v_cache,
+    const int64_t* __restrict__ slot_mapping, int H, int G, int D, int V,
+    int block_size, int interleaved) {
+  const int t = blockIdx.x;
+  const int hs = blockIdx.y;
+  const int lane = threadIdx.x;
+  const float pos = (float)positions[t];
+  const AT* src;
+  AT* dst;
+  const float* nw = nullptr;
+  const float* freq;
+  int n, npairs;
+  bool normed;
+  if (hs < H) {
+    src = q + (int64_t)t * ldq + (int64_t)hs * D;
+    dst = qo + ((int64_t)t * H + hs) * D;
+    n = D; npairs = n_rot; freq = freq_qk; nw = qw; normed = qw != nullptr;
+  } else {
+    const int64_t slot = slot_mapping[t];
+    if (slot < 0) return;
+    const int64_t blk = slot / block_size, off = slot % block_size;
+    if (hs < H + G) {
+      const int g = hs - H;
+      src = k + (int64_t)t * ldk + (int64_t)g * D;
+      dst = k_cache + ((blk * G + g) * block_size + off) * D;
+      n = D; npairs = n_rot; freq = freq_qk; nw = kw; normed = kw != nullptr;
+    } else {
+      const int g = hs - H - G;
+      src = v + (int64_t)t * ldv + (int64_t)g * V;
+      dst = v_cache + ((blk * G + g) * block_size + off) * V;
+      n = V; npairs = n_vrot; freq = freq_v; normed = false;
+    }
+  }
+  float rstd = 1.f;
+  if (normed) {
+    float ss = 0.f;
+    for (int i = lane; i < n; i += 64) {
+      const float a = Act<AT>::ld(src + i);
+      ss += a * a;
+    }
+    ss = wave_reduce_sum(ss);
+    rstd = 1.f / sqrtf(ss / (float)n + eps);
+  }
+  for (int i = lane; i < npairs; i += 64) {
+    const int d0 = interleaved ? 2 * i : i;
+    const int d1 = interleaved ? 2 * i + 1 : i + npairs;
+    float a = Act<AT>::ld(src + d0) * rstd;
+    float b = Act<AT>::ld(src + d1) * rstd;
+    if (normed) { a *= nw[d0]; b *= nw[d1]; }
+    float sn, cs;
+    sincosf(pos * freq[i], &sn, &cs);
+    Act<AT>::st(dst + d0, a * cs - b * sn);
+    Act<AT>::st(dst + d1, b * cs + a * sn);
+  }
+  for (int i = 2 * npairs + lane; i < n; i += 64) {
+    float a = Act<AT>::ld(src + i) * rstd;
+    if (normed) a *= nw[i];
+    Act<AT>::st(dst + i, a);
+  }
+}
+
+}  // namespace arks
+
+using namespace arks;
+
+extern "C" void arks_seq_token_shift(void* xs, void* xa, const void* x,
+                                     const void* w, void* state, const void* cu,
+                                     const void* seq_lens, const void* slots,
+                                     const void* token_seq, int T, int W,
+                                     int act_f32, hipStream_t stream) {
+  if (T == 0) return;
+  SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
+      (token_shift_kernel<AT>), dim3(T), dim3(256), 0, stream, (AT*)xs,
+      (AT*)xa, (const float*)x, (const float*)w, (float*)state, (const int*)cu,
+      (const int*)seq_lens, (const int*)slots, (const int*)token_seq, W));
+}
+
+extern "C" void arks_seq_gated_norm_residual(void* x, void* xa, const void* y,
+                                             const void* g, int64_t ldg,
+                                             const void* gb, const void* w,
+                                             float eps, int T, int W,
+                                             int act_f32, hipStream_t stream) {
+  if (T == 0) return;
+  SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
+      (gated_norm_residual_kernel<AT>), dim3(T), dim3(256), 0, stream,
+      (float*)x, (AT*)xa, (const AT*)y, (const AT*)g, ldg, (const float*)gb,
+      (const float*)w, eps, W));
+}
+
+extern "C" void arks_seq_rms_norm_f32(void* out, const void* x, const void* w,
+                                      const void* gate, int64_t ldg, float eps,
+                                      int T, int W, int act_f32,
+                                      hipStream_t stream) {
+  if (T == 0) return;
+  SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
+      (rms_norm_f32_kernel<AT>), dim3(T), dim3(256), 0, stream, (AT*)out,
+      (const float*)x, (const float*)w, (const AT*)gate, ldg, eps, W));
+}
+
+extern "C" void arks_seq_gelu_tanh(void* out, const void* x, int64_t ldx,
+                                   int64_t rows, int n, int act_f32,
+                                   hipStream_t stream) {
+  const int64_t total = rows * n;
+  if (total == 0) return;
+  SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
+      (gelu_tanh_kernel<AT>), dim3((unsigned)((total + 255) / 256)), dim3(256),
+      0, stream, (AT*)out, (const AT*)x, ldx, rows, n));
+}
+
+extern "C" void arks_seq_qk_norm_rope_cache(
+    void* qo, const void* q, const void* k, const void* v, int64_t ldq,
+    int64_t ldk, int64_t ldv, const void* qw, const void* kw, float eps,
+    const void* positions, const void* freq_qk, int n_rot, const void* freq_v,
+    int n_vrot, void* k_cache, void* v_cache, const void* slot_mapping, int T,
+    int H, int G, int D, int V, int block_size, int interleaved, int act_f32,
+    hipStream_t stream) {
+  if (T == 0) return;
+  SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
+      (qk_norm_rope_cache_kernel<AT>), dim3(T, H + 2 * G), dim3(64), 0, stream,
+      (AT*)qo, (const AT*)q, (const AT*)k, (const AT*)v, ldq, ldk, ldv,
+      (const float*)qw, (const float*)kw, eps, (const int64_t*)positions,
+      (const float*)freq_qk, n_rot, (const float*)freq_v, n_vrot, (AT*)k_cache,
+      (AT*)v_cache, (const int64_t*)slot_mapping, H, G, D, V, block_size,
+      interleaved));
+}

@@ -1,0 +1,101 @@
+// Lightning (linear) attention with one scalar decay per head:
+//   S_t = decay * S_{t-1} + k_t v_t^T,  o_t = S_t^T q_t,  q,k,v = silu(.)
+// S is a [D x V] fp32 matrix per head and sequence, kept in a slot-addressed
+// state tensor between steps.
+//
+// General kernel: one wave per (sequence, head, 64 value columns); lane c
+// owns column c of S in registers and walks the sequence's rows in order.
+// The row's silu(q), silu(k) are staged in LDS once per row for all lanes.
+#include "seq_common.h"
+
+namespace arks {
+
+template <typename AT, int DMAX>
+__global__ __launch_bounds__(64) void lightning_scan_kernel(
+    float* __restrict__ out, const AT* __restrict__ q, const AT* __restrict__ k,
+    const AT* __restrict__ v, int64_t ldq, int64_t ldk, int64_t ldv,
+    const float* __restrict__ decay, float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ seq_lens,
+    const int* __restrict__ slots, int H, int D, int V) {
+  __shared__ float q_s[2][DMAX];
+  __shared__ float k_s[2][DMAX];
+  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int col = blockIdx.z * 64 + lane;
+  const int a = cu[s], rows = cu[s + 1] - a;
+  if (rows == 0) return;
+  const int start = seq_lens[s] - rows;
+  const int slot = slots[s];
+  const bool live = col < V;
+  const float lam = decay[h];
+  float S[DMAX];
+  float* sp = state + (((int64_t)(slot < 0 ? 0 : slot) * H + h) * D) * V + col;
+  const bool has_state = start > 0 && slot >= 0 && live;
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d)
+    S[d] = (has_state && d < D) ? sp[(int64_t)d * V] : 0.f;
+  for (int r = 0; r < rows; ++r) {
+    const int t = a + r;
+    const int buf = r & 1;  // double buffer: one barrier per row
+    for (int d = lane; d < D; d += 64) {
+      q_s[buf][d] = silu_f(Act<AT>::ld(q + (int64_t)t * ldq + (int64_t)h * D + d));
+      k_s[buf][d] = silu_f(Act<AT>::ld(k + (int64_t)t * ldk + (int64_t)h * D + d));
+    }
+    const float vv =
+        live ? silu_f(Act<AT>::ld(v + (int64_t)t * ldv + (int64_t)h * V + col)) : 0.f;
+    __syncthreads();
+    float o = 0.f;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d) {
+      if (d < D) {
+        S[d] = lam * S[d] + k_s[buf][d] * vv;
+        o += S[d] * q_s[buf][d];
+      }
+    }
+    if (live) out[((int64_t)t * H + h) * V + col] = o;
+  }
+  if (slot >= 0 && live) {
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d)
+      if (d < D) sp[(int64_t)d * V] = S[d];
+  }
+}
+
+}  // namespace arks
+
+using namespace arks;
+
+template <typename AT>
+static int launch_lightning(float* out, const void* q, const void* k,
+                            const void* v, int64_t ldq, int64_t ldk,
+                            int64_t ldv, const float* decay, float* state,
+                            const int* cu, const int* seq_lens,
+                            const int* slots, int S, int H, int D, int V,
+                            hipStream_t stream) {
+  dim3 grid(S, H, (V + 63) / 64), block(64);
+#define LL(DM)                                                                 \
+  hipLaunchKernelGGL((lightning_scan_kernel<AT, DM>), grid, block, 0, stream,  \
+                     out, (const AT*)q, (const AT*)k, (const AT*)v, ldq, ldk,  \
+                     ldv, decay, state, cu, seq_lens, slots, H, D, V)
+  if (D <= 16) LL(16);
+  else if (D <= 32) LL(32);
+  else if (D <= 64) LL(64);
+  else if (D <= 128) LL(128);
+  else if (D <= 256) LL(256);
+  else return 1;
+#undef LL
+  return 0;
+}
+
+extern "C" int arks_seq_lightning_scan(
+    void* out, const void* q, const void* k, const void* v, int64_t ldq,
+    int64_t ldk, int64_t ldv, const void* decay, void* state, const void* cu,
+    const void* seq_lens, const void* slots, int S, int H, int D, int V,
+    int act_f32, hipStream_t stream) {
+  if (S == 0) return 0;
+  int rc = 0;
+  SEQ_DISPATCH_ACT(act_f32, rc = launch_lightning<AT>(
+      (float*)out, q, k, v, ldq, ldk, ldv, (const float*)decay, (float*)state,
+      (const int*)cu, (const int*)seq_lens, (const int*)slots, S, H, D, V,
+      stream));
+  return rc;
+}

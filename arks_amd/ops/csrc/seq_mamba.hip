@@ -1,0 +1,205 @@
+// Mamba1 mixer kernels: the short causal depthwise convolution (+ silu) with
+// its per-sequence history, and the selective scan
+//   S[c,n] <- exp(dt_c A[c,n]) S[c,n] + dt_c u_c B_n
+//   y_c = sum_n S[c,n] C_n + D_c u_c,   out = y * silu(z)
+// with dt = softplus(W_dt dt_raw + b) computed here in fp32, S fp32 in a
+// slot-addressed state tensor.
+#include "seq_common.h"
+
+namespace arks {
+
+constexpr int CONV_MAX_HIST = 8;  // taps - 1
+
+// One block per row, threads over channels. Inputs before the step's first
+// row come from the sequence's stored history (zeros at position 0). The
+// history is replaced by conv_state_update_kernel in a later launch, so
+// every reader here sees the old one.
+template <typename AT>
+__global__ __launch_bounds__(256) void causal_conv_silu_kernel(
+    AT* __restrict__ out, const AT* __restrict__ x, int64_t ldx,
+    const float* __restrict__ w, const float* __restrict__ bias,
+    const float* __restrict__ state, const int* __restrict__ cu,
+    const int* __restrict__ seq_lens, const int* __restrict__ slots,
+    const int* __restrict__ token_seq, int C, int taps) {
+  const int t = blockIdx.x;
+  const SeqRow r = seq_row(t, token_seq, cu, seq_lens, slots);
+  const int i = t - r.first_row;
+  const bool has_state = r.start > 0 && r.slot >= 0;
+  const float* hist = state + (int64_t)(r.slot < 0 ? 0 : r.slot) * (taps - 1) * C;
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
+    float acc = bias[c];
+    for (int j = 0; j < taps; ++j) {
+      const int src = i - (taps - 1 - j);
+      float xv;
+      if (src >= 0)
+        xv = Act<AT>::ld(x + (int64_t)(r.first_row + src) * ldx + c);
+      else
+        xv = has_state ? hist[(int64_t)(src + taps - 1) * C + c] : 0.f;
+      acc += w[(int64_t)c * taps + j] * xv;
+    }
+    Act<AT>::st(out + (int64_t)t * C + c, silu_f(acc));
+  }
+}
+
+// New history of a sequence = the last taps-1 inputs after this step: rows
+// of this step where there are enough, older history shifted up otherwise.
+// One thread per (sequence, channel) reads all it needs before it writes.
+template <typename AT>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(
+    float* __restrict__ state, const AT* __restrict__ x, int64_t ldx,
+    const int* __restrict__ cu, const int* __restrict__ seq_lens,
+    const int* __restrict__ slots, int C, int taps) {
+  const int s = blockIdx.x;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  const int a = cu[s], rows = cu[s + 1] - a;
+  const int slot = slots[s];
+  if (c >= C || rows == 0 || slot < 0) return;
+  const int start = seq_lens[s] - rows;
+  const int nh = taps - 1;
+  float* hist = state + (int64_t)slot * nh * C + c;
+  float nv[CONV_MAX_HIST];
+#pragma unroll
+  for (int i = 0; i < CONV_MAX_HIST; ++i) {
+    if (i < nh) {
+      const int src = rows - nh + i;  // index into this step's rows
+      if (src >= 0)
+        nv[i] = Act<AT>::ld(x + (int64_t)(a + src) * ldx + c);
+      else
+        nv[i] = start > 0 ? hist[(int64_t)(src + nh) * C] : 0.f;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < CONV_MAX_HIST; ++i)
+    if (i < nh) hist[(int64_t)i * C] = nv[i];
+}
+
+// General selective scan: 16 lanes per channel (4 channels per wave), lane
+// ln owns states n = ln + 16 i. Rows are walked in order; dt's projection
+// and the output sum are reduced over the 16 lanes.
+template <typename AT, int NPT>
+__global__ __launch_bounds__(64) void selective_scan_kernel(
+    AT* __restrict__ out, const AT* __restrict__ u, const AT* __restrict__ dbc,
+    int64_t ldd, const AT* __restrict__ z, int64_t ldz,
+    const float* __restrict__ dt_w, const float* __restrict__ dt_b,
+    const float* __restrict__ A, const float* __restrict__ Dp,
+    float* __restrict__ state, const int* __restrict__ cu,
+    const int* __restrict__ seq_lens, const int* __restrict__ slots, int C,
+    int N, int R) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * 4 + threadIdx.x / 16;
+  const int ln = threadIdx.x % 16;
+  const int a = cu[s], rows = cu[s + 1] - a;
+  if (rows == 0) return;
+  const bool live = c < C;
+  const int cc = live ? c : C - 1;  // keep the whole wave in the shuffles
+  const int start = seq_lens[s] - rows;
+  const int slot = slots[s];
+  const bool has_state = start > 0 && slot >= 0;
+  float* sp = state + ((int64_t)(slot < 0 ? 0 : slot) * C + cc) * N;
+  float S[NPT], Av[NPT];
+#pragma unroll
+  for (int i = 0; i < NPT; ++i) {
+    const int n = ln + 16 * i;
+    S[i] = (has_state && n < N) ? sp[n] : 0.f;
+    Av[i] = n < N ? A[(int64_t)cc * N + n] : 0.f;
+  }
+  const float dtb = dt_b[cc], dd = Dp[cc];
+  const float* wr = dt_w + (int64_t)cc * R;
+  for (int r = 0; r < rows; ++r) {
+    const int t = a + r;
+    const AT* drow = dbc + (int64_t)t * ldd;
+    float dtp = 0.f;
+    for (int j = ln; j < R; j += 16) dtp += wr[j] * Act<AT>::ld(drow + j);
+    const float dt = softplus_f(group16_reduce_sum(dtp) + dtb);
+    const float xv = Act<AT>::ld(u + (int64_t)t * C + cc);
+    const float dx = dt * xv;
+    float y = 0.f;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+      const int n = ln + 16 * i;
+      if (n < N) {
+        const float Bn = Act<AT>::ld(drow + R + n);
+        const float Cn = Act<AT>::ld(drow + R + N + n);
+        S[i] = expf(dt * Av[i]) * S[i] + dx * Bn;
+        y += S[i] * Cn;
+      }
+    }
+    y = group16_reduce_sum(y) + dd * xv;
+    if (ln == 0 && live) {
+      const float zv = Act<AT>::ld(z + (int64_t)t * ldz + c);
+      Act<AT>::st(out + (int64_t)t * C + c, y * silu_f(zv));
+    }
+  }
+  if (slot >= 0 && live) {
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+      const int n = ln + 16 * i;
+      if (n < N) sp[n] = S[i];
+    }
+  }
+}
+
+}  // namespace arks
+
+using namespace arks;
+
+extern "C" int arks_seq_causal_conv_silu(
+    void* out, const void* x, int64_t ldx, const void* w, const void* bias,
+    void* state, const void* cu, const void* seq_lens, const void* slots,
+    const void* token_seq, int T, int S, int C, int taps, int act_f32,
+    hipStream_t stream) {
+  if (taps - 1 > CONV_MAX_HIST || taps < 1) return 1;
+  if (T == 0) return 0;
+  const int cb = (C + 255) / 256;
+  SEQ_DISPATCH_ACT(act_f32, {
+    hipLaunchKernelGGL((causal_conv_silu_kernel<AT>), dim3(T, cb), dim3(256), 0,
+                       stream, (AT*)out, (const AT*)x, ldx, (const float*)w,
+                       (const float*)bias, (const float*)state, (const int*)cu,
+                       (const int*)seq_lens, (const int*)slots,
+                       (const int*)token_seq, C, taps);
+    if (taps > 1)
+      hipLaunchKernelGGL((conv_state_update_kernel<AT>), dim3(S, cb), dim3(256),
+                         0, stream, (float*)state, (const AT*)x, ldx,
+                         (const int*)cu, (const int*)seq_lens,
+                         (const int*)slots, C, taps);
+  });
+  return 0;
+}
+
+template <typename AT>
+static int launch_scan(void* out, const void* u, const void* dbc, int64_t ldd,
+                       const void* z, int64_t ldz, const float* dt_w,
+                       const float* dt_b, const float* A, const float* Dp,
+                       float* state, const int* cu, const int* seq_lens,
+                       const int* slots, int S, int C, int N, int R,
+                       hipStream_t stream) {
+  dim3 grid((C + 3) / 4, S), block(64);
+#define SS(NP)                                                                \
+  hipLaunchKernelGGL((selective_scan_kernel<AT, NP>), grid, block, 0, stream, \
+                     (AT*)out, (const AT*)u, (const AT*)dbc, ldd,             \
+                     (const AT*)z, ldz, dt_w, dt_b, A, Dp, state, cu,         \
+                     seq_lens, slots, C, N, R)
+  if (N <= 16) SS(1);
+  else if (N <= 32) SS(2);
+  else if (N <= 64) SS(4);
+  else if (N <= 128) SS(8);
+  else if (N <= 256) SS(16);
+  else return 1;
+#undef SS
+  return 0;
+}
+
+extern "C" int arks_seq_selective_scan(
+    void* out, const void* u, const void* dbc, int64_t ldd, const void* z,
+    int64_t ldz, const void* dt_w, const void* dt_b, const void* A,
+    const void* Dp, void* state, const void* cu, const void* seq_lens,
+    const void* slots, int S, int C, int N, int R, int act_f32,
+    hipStream_t stream) {
+  if (S == 0) return 0;
+  int rc = 0;
+  SEQ_DISPATCH_ACT(act_f32, rc = launch_scan<AT>(
+      out, u, dbc, ldd, z, ldz, (const float*)dt_w, (const float*)dt_b,
+      (const float*)A, (const float*)Dp, (float*)state, (const int*)cu,
+      (const int*)seq_lens, (const int*)slots, S, C, N, R, stream));
+  return rc;
+}

@@ -325,3 +325,229 @@ def gumbel_sample(
 
 def softmax_scale(head_dim: int) -> float:
     return 1.0 / math.sqrt(head_dim)
+
+
+# ----------------------------------------------------------------------
+# Sequence-state ops (token shift, gated output norm, sink attention with
+# rotated values, lightning linear attention, mamba1 conv + selective scan).
+# Shared conventions: rows of a step are packed [T, ...]; cu_seqlens[s] is
+# the first row of sequence s, seq_lens[s] its length INCLUDING this step's
+# rows (so its first new position is seq_lens[s] - rows), state_slots[s] the
+# row of every per-sequence state tensor (-1 = padding: read zeros, write
+# nothing). A sequence whose first new position is 0 starts from zero state
+# whatever its slot holds, so slots are reused without clearing.
+# ----------------------------------------------------------------------
+def _seq_spans(cu_seqlens, seq_lens, state_slots):
+    cu = cu_seqlens.tolist()
+    sl = seq_lens.tolist()
+    slots = state_slots.tolist()
+    for s in range(len(sl)):
+        a, b = cu[s], cu[s + 1]
+        if b > a:
+            yield a, b, sl[s] - (b - a), slots[s]
+
+
+def token_shift(x, shift_w, prev_state, cu_seqlens, seq_lens, state_slots,
+                out_dtype):
+    """xs[t] = x[t] + (x[t-1] - x[t]) * shift_w, x[-1] of a sequence being
+    the last row of its previous step (prev_state) or zero at position 0.
+    Stores each sequence's last row into prev_state. Returns (xs, x) cast
+    to out_dtype."""
+    xs = torch.empty_like(x)
+    w = shift_w.float()
+    for a, b, start, slot in _seq_spans(cu_seqlens, seq_lens, state_slots):
+        first = (prev_state[slot].clone() if start > 0 and slot >= 0
+                 else torch.zeros_like(x[a]))
+        prev = torch.cat([first[None], x[a:b - 1]], 0)
+        xs[a:b] = x[a:b] + (prev - x[a:b]) * w
+        if slot >= 0:
+            prev_state[slot] = x[b - 1]
+    return xs.to(out_dtype), x.to(out_dtype)
+
+
+def gated_norm_residual(x, y, gate, gate_bias, weight, eps, out_dtype=None):
+    """x += rmsnorm(y * sigmoid(gate + gate_bias)) * weight, everything in
+    fp32, x updated in place; gate None = no gate. Returns x cast to
+    out_dtype (or None)."""
+    z = y.float()
+    if gate is not None:
+        z = z * torch.sigmoid(gate.float() + gate_bias.float())
+    r = z * torch.rsqrt(z.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    x += r
+    return x.to(out_dtype) if out_dtype is not None else None
+
+
+def rms_norm_f32(x, weight, eps, out_dtype):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+            * weight.float()).to(out_dtype)
+
+
+def _rotate_pairs(x, angles, interleaved: bool):
+    """x [..., 2*P] turned pairwise by angles [..., P] (fp32)."""
+    c, s = torch.cos(angles), torch.sin(angles)
+    out = torch.empty_like(x)
+    if interleaved:
+        u, w = x[..., 0::2], x[..., 1::2]
+        out[..., 0::2] = u * c - w * s
+        out[..., 1::2] = w * c + u * s
+    else:
+        P = x.shape[-1] // 2
+        u, w = x[..., :P], x[..., P:]
+        out[..., :P] = u * c - w * s
+        out[..., P:] = w * c + u * s
+    return out
+
+
+def qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
+                       inv_freq_qk, inv_freq_v, k_cache, v_cache,
+                       slot_mapping, interleaved=True):
+    """q [T,H,D], k [T,G,D], v [T,G,V]: per-head RMS norm of q and k (weights
+    or None), rotary on their first 2*len(inv_freq_qk) dims, values turned by
+    their own position over all V dims (inv_freq_v None = values stored
+    plain); k and v go to the paged cache. Returns q (fp32 math, q.dtype)."""
+    pos = positions.float()
+
+    def prep(t, w, inv_freq):
+        tf = t.float()
+        if w is not None:
+            tf = tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        if inv_freq is not None and inv_freq.numel():
+            rd = 2 * inv_freq.numel()
+            ang = pos[:, None, None] * inv_freq.float()[None, None, :]
+            tf = torch.cat([_rotate_pairs(tf[..., :rd], ang, interleaved),
+                            tf[..., rd:]], -1)
+        return tf
+
+    qo = prep(q, q_norm_w, inv_freq_qk).to(q.dtype)
+    ko = prep(k, k_norm_w, inv_freq_qk).to(k_cache.dtype)
+    vo = prep(v, None, inv_freq_v).to(v_cache.dtype)
+    bs = k_cache.shape[2]
+    ok = slot_mapping >= 0
+    blk = (slot_mapping[ok] // bs).long()
+    off = (slot_mapping[ok] % bs).long()
+    k_cache[blk, :, off] = ko[ok]
+    v_cache[blk, :, off] = vo[ok]
+    return qo
+
+
+def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
+                         cu_seqlens, scale, sink=True, inv_freq_v=None,
+                         interleaved=True):
+    """Causal attention of packed new rows over each sequence's paged keys.
+    sink=True adds a value-less key of score 0 to every softmax (one more
+    in the denominator). inv_freq_v: each row's output is turned back by its
+    own position over the value dims. q [T,H,D] -> [T,H,V] in q.dtype."""
+    T, H, D = q.shape
+    G, bs, V = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    out = torch.zeros(T, H, V, dtype=torch.float32)
+    cu = cu_seqlens.tolist()
+    sl = seq_lens.tolist()
+    for s in range(len(sl)):
+        a, b = cu[s], cu[s + 1]
+        n, L = b - a, sl[s]
+        if n == 0:
+            continue
+        nb = (L + bs - 1) // bs
+        pages = block_tables[s, :nb].long()
+        K = k_cache[pages].permute(1, 0, 2, 3).reshape(G, nb * bs, D)[:, :L].float()
+        Vv = v_cache[pages].permute(1, 0, 2, 3).reshape(G, nb * bs, V)[:, :L].float()
+        K = K.repeat_interleave(H // G, 0)
+        Vv = Vv.repeat_interleave(H // G, 0)
+        qs = q[a:b].float().permute(1, 0, 2)  # [H, n, D]
+        sc = torch.matmul(qs, K.transpose(1, 2)) * scale  # [H, n, L]
+        qpos = torch.arange(L - n, L)
+        mask = torch.arange(L)[None, :] > qpos[:, None]
+        sc = sc.masked_fill(mask[None], float("-inf"))
+        m = sc.amax(-1, keepdim=True)
+        if sink:
+            m = m.clamp(min=0.0)
+        e = torch.exp(sc - m)
+        den = e.sum(-1, keepdim=True)
+        if sink:
+            den = den + torch.exp(-m)
+        o = torch.matmul(e / den, Vv).permute(1, 0, 2)  # [n, H, V]
+        if inv_freq_v is not None:
+            ang = -qpos.float()[:, None, None] * inv_freq_v.float()[None, None, :]
+            o = _rotate_pairs(o, ang, interleaved)
+        out[a:b] = o
+    return out.to(q.dtype)
+
+
+def lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots):
+    """Per head S <- decay*S + silu(k) silu(v)^T, o = S^T silu(q); q,k
+    [T,H,D], v [T,H,V], state [slots,H,D,V] fp32 (updated). -> o fp32
+    [T,H,V]."""
+    T, H, D = q.shape
+    V = v.shape[-1]
+    F = torch.nn.functional
+    qf, kf, vf = F.silu(q.float()), F.silu(k.float()), F.silu(v.float())
+    out = torch.zeros(T, H, V, dtype=torch.float32)
+    lam = decay.float()[:, None, None]
+    for a, b, start, slot in _seq_spans(cu_seqlens, seq_lens, state_slots):
+        S = (state[slot].clone() if start > 0 and slot >= 0
+             else torch.zeros(H, D, V))
+        for t in range(a, b):
+            S = lam * S + kf[t][:, :, None] * vf[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        if slot >= 0:
+            state[slot] = S
+    return out
+
+
+def gated_rmsnorm(o, weight, gate, eps, out_dtype):
+    """rmsnorm(o) * weight * sigmoid(gate) over the last dim."""
+    of = o.float()
+    y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps) * weight.float()
+    return (y * torch.sigmoid(gate.float())).to(out_dtype)
+
+
+def causal_conv_silu(x, weight, bias, state, cu_seqlens, seq_lens,
+                     state_slots):
+    """Depthwise causal conv over time then silu. x [T,C]; weight [C,taps]
+    (last column = current row); state [slots,taps-1,C] fp32 holds each
+    sequence's last taps-1 inputs (updated)."""
+    T, C = x.shape
+    taps = weight.shape[1]
+    xf = x.float()
+    out = torch.empty(T, C, dtype=torch.float32)
+    for a, b, start, slot in _seq_spans(cu_seqlens, seq_lens, state_slots):
+        hist = (state[slot].clone() if start > 0 and slot >= 0 and taps > 1
+                else torch.zeros(taps - 1, C))
+        full = torch.cat([hist, xf[a:b]], 0)  # [taps-1+n, C]
+        n = b - a
+        acc = bias.float()[None, :].expand(n, C).clone()
+        for j in range(taps):
+            acc += full[j:j + n] * weight.float()[:, j][None, :]
+        out[a:b] = acc
+        if slot >= 0 and taps > 1:
+            state[slot] = full[n:]
+    return torch.nn.functional.silu(out).to(x.dtype)
+
+
+def selective_scan(u, dbc, z, dt_w, dt_b, A, Dp, state, cu_seqlens,
+                   seq_lens, state_slots):
+    """Mamba1 recurrence. u [T,C] (conv output), dbc [T,R+2N] = [dt|B|C],
+    z [T,C] gate, dt_w [C,R], A [C,N] (negative), state [slots,C,N] fp32
+    (updated). -> y [T,C] in u.dtype, y = (S.C + D u) * silu(z)."""
+    T, C = u.shape
+    R = dt_w.shape[1]
+    N = A.shape[1]
+    uf, zf, df = u.float(), z.float(), dbc.float()
+    dt = torch.nn.functional.softplus(df[:, :R] @ dt_w.float().t() + dt_b.float())
+    Bm, Cm = df[:, R:R + N], df[:, R + N:R + 2 * N]
+    out = torch.empty(T, C, dtype=torch.float32)
+    Af = A.float()
+    for a, b, start, slot in _seq_spans(cu_seqlens, seq_lens, state_slots):
+        S = (state[slot].clone() if start > 0 and slot >= 0
+             else torch.zeros(C, N))
+        for t in range(a, b):
+            S = torch.exp(dt[t][:, None] * Af) * S + (dt[t] * uf[t])[:, None] * Bm[t][None, :]
+            out[t] = S @ Cm[t] + Dp.float() * uf[t]
+        if slot >= 0:
+            state[slot] = S
+    return (out * torch.nn.functional.silu(zf)).to(u.dtype)
+
+
+def gelu_tanh(x):
+    return torch.nn.functional.gelu(x.float(), approximate="tanh").to(x.dtype)

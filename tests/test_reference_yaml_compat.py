@@ -23,7 +23,8 @@ KIND_MAP = {
 }
 
 pytestmark = pytest.mark.skipif(
-    not os.path.isdir(REF), reason="reference checkout not present"
+    not os.path.isdir(os.path.join(REF, "examples")),
+    reason="reference checkout not present"
 )
 
 
