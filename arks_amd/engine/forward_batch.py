@@ -2,7 +2,7 @@
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import torch
 
@@ -35,6 +35,11 @@ class ForwardBatch:
     state_slots: torch.Tensor | None = None  # [num_seqs] int32
     token_seq: torch.Tensor | None = None  # [total_tokens] int32
     max_q_len: int = 0
+    # host copies of the per-sequence total lengths (None inside a captured
+    # decode graph) and the per-step cache of kernel work lists built from
+    # them, keyed by head layout
+    kv_lens_list: list[int] | None = None
+    tile_cache: dict = field(default_factory=dict)
 
     @property
     def num_tokens(self) -> int:

@@ -349,6 +349,7 @@ class ModelRunner:
             seq_lens=torch.tensor(seq_lens, dtype=torch.int32, device=dev),
             **(dict(cu_seqlens=torch.arange(len(sb.seqs) + 1, dtype=torch.int32,
                                             device=dev),
+                    seq_lens_list=[1] * len(sb.seqs),
                     **self._state_fields(sb.seqs, [1] * len(sb.seqs)))
                if self.seq_state else {}),
         )
@@ -366,6 +367,7 @@ class ModelRunner:
             token_seq=torch.from_numpy(np.repeat(
                 np.arange(len(seqs), dtype=np.int32), q_lens)).to(dev),
             max_q_len=max(q_lens),
+            kv_lens_list=[s.num_cached_tokens for s in seqs],
         )
 
     # ---------------- hipGraph decode ----------------

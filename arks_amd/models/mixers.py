@@ -88,6 +88,22 @@ class SinkRotaryAttention(nn.Module):
         return {"k": ("paged", (self.G, block_size, self.D), dtype),
                 "v": ("paged", (self.G, block_size, self.V), dtype)}
 
+    def _tiles(self, batch: ForwardBatch, q):
+        """Work lists of the MFMA kernels: host-built once per step and head
+        layout (batch.tile_cache), shared by every layer of that layout.
+        None where the general kernel runs (CPU, float32, other sizes,
+        graph-captured decode steps, whose lengths are not known on the
+        host)."""
+        if (not q.is_cuda or q.dtype != torch.bfloat16 or self.D != self.V
+                or batch.kv_lens_list is None):
+            return None
+        key = (self.H, self.G, self.D)
+        if key not in batch.tile_cache:
+            batch.tile_cache[key] = ops.sink_attention_tiles(
+                batch.seq_lens_list, batch.kv_lens_list, self.H, self.G,
+                self.D, q.device)
+        return batch.tile_cache[key]
+
     def forward(self, xs, batch: ForwardBatch, cache: dict) -> torch.Tensor:
         T = xs.shape[0]
         H, G, D, V = self.H, self.G, self.D, self.V
@@ -102,7 +118,8 @@ class SinkRotaryAttention(nn.Module):
         out = ops.attention_sink_paged(
             q, cache["k"], cache["v"], batch.block_tables, batch.seq_lens,
             batch.cu_seqlens, batch.token_seq, self.scale, self.sink,
-            self.inv_freq_v, self.interleaved, batch.max_q_len)
+            self.inv_freq_v, self.interleaved, batch.max_q_len,
+            batch.positions, self._tiles(batch, q))
         return linear(out.view(T, H * V), self.o)
 
 

@@ -145,7 +145,8 @@ EXTEND2_MIN_QLEN = 97
 
 
 def build_extend_tiles(q_lens: list[int], kv_lens: list[int] | None,
-                       kv_fp8: bool, device, num_q_heads: int = 32):
+                       kv_fp8: bool, device, num_q_heads: int = 32,
+                       ladder: bool = True, flash_decode: bool = True):
     """Per-seq routing for the extend dispatcher:
     (tiles64, tiles256 [n,4], decode_rows, combine_table, ws_rows).
 
@@ -165,9 +166,9 @@ def build_extend_tiles(q_lens: list[int], kv_lens: list[int] | None,
     kvl = kv_lens if kv_lens is not None else q_lens
     for i, n in enumerate(q_lens):
         off = kvl[i] - n
-        if n == 1:
+        if n == 1 and flash_decode:
             dec.append(i)
-        elif kv_fp8 or n < EXTEND2_MIN_QLEN:
+        elif kv_fp8 or n < EXTEND2_MIN_QLEN or not ladder:
             for q0 in range(0, n, PREFILL_QTILE):
                 t64.append((i, q0, min(kvl[i], off + q0 + PREFILL_QTILE)))
         else:
@@ -231,18 +232,23 @@ def build_extend_tiles(q_lens: list[int], kv_lens: list[int] | None,
 def attention_extend_paged(
     q, k_cache, v_cache, block_tables, kv_lens, cu_seqlens_q,
     q_lens: list[int], scale: float, window: int = 0, tiles=None,
+    sink: bool = False, native=None,
 ):
     """Causal attention of packed NEW tokens over each sequence's full paged
     KV history (cached prefix + new tokens already written by
     reshape_and_cache). The prefix-caching / chunked-prefill attention path.
     q_lens is the host-side per-seq new-token count (tile grid without a
     D2H sync); kv_lens is the device int32 total kv length per seq.
-    window > 0 = sliding-window attention.
+    window > 0 = sliding-window attention. sink: every softmax also holds a
+    value-less key of score 0. native: the extension whose build of these
+    kernels runs (default: arks_amd_C).
 
     Dispatch: big chunks run the 8-wave 32x32-MFMA ladder kernel
     (attn_extend2.hip, 256-row q tiles); small chunks and fp8-KV runs use
     the 4-wave 64-row kernel."""
     if q.is_cuda:
+        C = native if native is not None else _native()
+        sink = 1 if sink else 0
         out = torch.empty(
             (q.shape[0], q.shape[1], q.shape[2]), dtype=q.dtype, device=q.device
         )
@@ -260,18 +266,18 @@ def attention_extend_paged(
                 )
             else:
                 ws = q.new_empty(0, dtype=torch.float32)
-            _native().attention_extend_paged2(
+            C.attention_extend_paged2(
                 out, q, k_cache, v_cache, block_tables, kv_lens, cu_seqlens_q,
-                t256, ws, scale, window,
+                t256, ws, scale, window, sink,
             )
             if ctab.numel():
-                _native().attention_extend2_combine(
+                C.attention_extend2_combine(
                     out, ws, ctab, cu_seqlens_q, scale,
                 )
         if t64.numel():
-            _native().attention_extend_paged(
+            C.attention_extend_paged(
                 out, q, k_cache, v_cache, block_tables, kv_lens, cu_seqlens_q,
-                t64, scale, window,
+                t64, scale, window, sink,
             )
         if drows is not None:
             dq = q[drows].contiguous()
@@ -279,6 +285,7 @@ def attention_extend_paged(
                 dq, k_cache, v_cache,
                 block_tables[dseqs].contiguous(),
                 kv_lens[dseqs].contiguous(), scale, window=window,
+                sink=bool(sink), native=C,
             )
             out[drows] = dout
         return out
@@ -304,8 +311,10 @@ def decode_num_partitions(num_seqs: int, num_kv_heads: int, max_blocks: int) -> 
 def attention_decode_paged(
     q, k_cache, v_cache, block_tables, seq_lens, scale: float,
     num_partitions: int | None = None, part_out=None, window: int = 0,
+    sink: bool = False, native=None,
 ):
     if q.is_cuda:
+        C = native if native is not None else _native()
         out = torch.empty(
             (q.shape[0], q.shape[1], q.shape[2]), dtype=q.dtype, device=q.device
         )
@@ -322,9 +331,9 @@ def attention_decode_paged(
             )
         elif part_out is None:
             part_out = q.new_empty(0, dtype=torch.float32)
-        _native().attention_decode_paged(
+        C.attention_decode_paged(
             out, q, k_cache, v_cache, block_tables, seq_lens, scale,
-            part_out, num_partitions, window,
+            part_out, num_partitions, window, 1 if sink else 0,
         )
         return out
     return ref.attention_decode_paged(
@@ -642,12 +651,54 @@ def qk_norm_rope_cache(q, k, v, q_norm_w, k_norm_w, eps, positions,
                                   slot_mapping, interleaved)
 
 
+# head sizes the MFMA kernels are built for (q/k size == value size)
+_MFMA_HEAD_DIMS = (32, 64, 96, 128, 256)
+_MFMA_LADDER_DIMS = (64, 128)  # 256-row ladder + flash-decode kernels
+
+
+def sink_attention_tiles(q_lens, kv_lens, num_q_heads, num_kv_heads,
+                         head_dim, device):
+    """Work lists of the MFMA attention kernels for one step and one head
+    layout (build once per step, reuse in every layer of that layout)."""
+    big = head_dim in _MFMA_LADDER_DIMS
+    return build_extend_tiles(
+        q_lens, kv_lens, False, device, num_q_heads=num_q_heads, ladder=big,
+        flash_decode=big and num_q_heads // num_kv_heads <= 8)
+
+
 def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
                          cu_seqlens, token_seq, scale, sink=True,
-                         inv_freq_v=None, interleaved=True, max_q_len=0):
+                         inv_freq_v=None, interleaved=True, max_q_len=0,
+                         positions=None, tiles=None):
+    """Causal attention of packed rows over paged keys with an optional
+    sink and position-turned values (see ref.attention_sink_paged). bf16
+    rows with equal q/k and value head sizes the MFMA kernels are built for
+    run those (then a pass that turns each row's output back); anything
+    else — float32 rows, other sizes — runs the general kernel."""
     if q.is_cuda:
-        T, H, _ = q.shape
+        T, H, D = q.shape
         V = v_cache.shape[3]
+        G = k_cache.shape[1]
+        fast = (q.dtype == torch.bfloat16 and D == V and k_cache.shape[2] == 16)
+        if (fast and max_q_len == 1 and T == seq_lens.shape[0]
+                and D in _MFMA_LADDER_DIMS and H // G <= 8):
+            # one row per sequence: the flash-decode kernel needs no host
+            # work list, so it also runs inside a captured decode graph
+            out = attention_decode_paged(
+                q, k_cache, v_cache, block_tables, seq_lens, scale,
+                sink=sink, native=_native_seq())
+            if inv_freq_v is not None:
+                _native_seq().unrotate_rows(out, positions, inv_freq_v,
+                                            interleaved)
+            return out
+        if fast and tiles is not None and D in _MFMA_HEAD_DIMS:
+            out = attention_extend_paged(
+                q, k_cache, v_cache, block_tables, seq_lens, cu_seqlens,
+                None, scale, tiles=tiles, sink=sink, native=_native_seq())
+            if inv_freq_v is not None:
+                _native_seq().unrotate_rows(out, positions, inv_freq_v,
+                                            interleaved)
+            return out
         out = torch.empty((T, H, V), dtype=q.dtype, device=q.device)
         _native_seq().attention_sink_paged(
             out, q, k_cache, v_cache, block_tables, seq_lens, cu_seqlens,

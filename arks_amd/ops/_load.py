@@ -14,7 +14,18 @@ from .build import built_so_path
 
 
 
+_loaded: dict = {}
+
+
+def __getattr__(attr: str):
+    if attr == "C":  # the main extension, loaded on first use
+        return load("arks_amd_C")
+    raise AttributeError(attr)
+
+
 def load(name: str):
+    if name in _loaded:
+        return _loaded[name]
     so = built_so_path(name)
     if so is None:
         raise ImportError(
@@ -24,4 +35,5 @@ def load(name: str):
     spec = importlib.util.spec_from_file_location(name, so)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
+    _loaded[name] = mod
     return mod

@@ -41,6 +41,10 @@ SEQ_SOURCES = [
     os.path.join(CSRC, "seq_bindings.cpp"),
     os.path.join(CSRC, "seq_elementwise.hip"),
     os.path.join(CSRC, "seq_attention.hip"),
+    # the framework's MFMA paged-attention kernels, built with the sink
+    os.path.join(CSRC, "attn_extend.hip"),
+    os.path.join(CSRC, "attn_extend2.hip"),
+    os.path.join(CSRC, "attn_decode.hip"),
     os.path.join(CSRC, "seq_lightning.hip"),
     os.path.join(CSRC, "seq_mamba.hip"),
 ]

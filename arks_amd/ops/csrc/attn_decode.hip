@@ -71,7 +71,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const int* __restrict__ block_tables,  // [S, max_blocks]
     const int* __restrict__ seq_lens,      // [S]
     const float scale, const int num_kv_heads, const int max_blocks,
-    const int64_t q_stride, const int window) {
+    const int64_t q_stride, const int window, const int sink) {
   constexpr int NUM_WAVES = 4;
   constexpr int STEPS = HEAD_DIM / 32;   // QK^T contraction steps
   constexpr int CHUNKS = HEAD_DIM / 16;  // PV output dim chunks
@@ -395,6 +395,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
         mf = mn;
       }
       if (nparts == 1) {
+        // sink: one more key of score 0 and no value in the denominator
+        if (sink) lf += __expf(-mf);
         const float inv = lf > 0.f ? 1.f / lf : 0.f;
         bf16* op = out +
                    ((int64_t)seq * num_q_heads + kvh * GQ + g) * HEAD_DIM +
@@ -432,7 +434,7 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
     bf16* __restrict__ out,             // [S, Hq, D]
     const float* __restrict__ part_out,  // [S, Hkv, P, GQ, D+2]
     const int* __restrict__ seq_lens, const int num_q_heads,
-    const int num_kv_heads, const int nparts) {
+    const int num_kv_heads, const int nparts, const int sink) {
   constexpr int E = HEAD_DIM / 16;
   const int seq = blockIdx.x;
   const int h = blockIdx.y;
@@ -466,6 +468,7 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
       af[e] = af[e] * a1 + pp[lane16 * E + e] * a2;
     mf = mn;
   }
+  if (sink) lf += __expf(-mf);
   const float inv = lf > 0.f ? 1.f / lf : 0.f;
   bf16* op = out + ((int64_t)seq * num_q_heads + h) * HEAD_DIM + lane16 * E;
   if constexpr (E == 8) {
@@ -486,7 +489,7 @@ void launch_decode_gq(bf16* out, float* part_out, const bf16* q,
                       const bf16* kc, const bf16* vc, const int* bt,
                       const int* sl, float scale, int num_seqs,
                       int num_kv_heads, int gq, int max_blocks, int nparts,
-                      int64_t q_stride, bool kv_fp8, int window,
+                      int64_t q_stride, bool kv_fp8, int window, int sink,
                       hipStream_t stream) {
   dim3 grid(num_kv_heads, num_seqs, nparts), block(256);
 #define ARKS_CASE(G)                                                          \
@@ -494,11 +497,13 @@ void launch_decode_gq(bf16* out, float* part_out, const bf16* q,
     if (kv_fp8) {                                                             \
       hipLaunchKernelGGL((attn_decode_kernel<HEAD_DIM, G, true>), grid,       \
                          block, 0, stream, out, part_out, q, kc, vc, bt, sl,  \
-                         scale, num_kv_heads, max_blocks, q_stride, window);  \
+                         scale, num_kv_heads, max_blocks, q_stride, window,   \
+                         sink);                                               \
     } else {                                                                  \
       hipLaunchKernelGGL((attn_decode_kernel<HEAD_DIM, G, false>), grid,      \
                          block, 0, stream, out, part_out, q, kc, vc, bt, sl,  \
-                         scale, num_kv_heads, max_blocks, q_stride, window);  \
+                         scale, num_kv_heads, max_blocks, q_stride, window,   \
+                         sink);                                               \
     }                                                                         \
     break;
   switch (gq) {
@@ -518,7 +523,7 @@ void launch_decode_gq(bf16* out, float* part_out, const bf16* q,
     dim3 cgrid(num_seqs, num_kv_heads * gq), cblock(64);
     hipLaunchKernelGGL((attn_decode_combine_kernel<HEAD_DIM>), cgrid, cblock,
                        0, stream, out, part_out, sl, num_kv_heads * gq,
-                       num_kv_heads, nparts);
+                       num_kv_heads, nparts, sink);
   }
 }
 
@@ -534,19 +539,19 @@ extern "C" void arks_attn_decode_paged(void* out, void* part_out, const void* q,
                                        int num_kv_heads, int head_dim,
                                        int max_blocks, int nparts,
                                        int64_t q_stride, int kv_fp8, int window,
-                                       hipStream_t stream) {
+                                       int sink, hipStream_t stream) {
   const int gq = num_q_heads / num_kv_heads;
   if (head_dim == 128) {
     launch_decode_gq<128>((bf16*)out, (float*)part_out, (const bf16*)q,
                           (const bf16*)k_cache, (const bf16*)v_cache,
                           (const int*)block_tables, (const int*)seq_lens,
                           scale, num_seqs, num_kv_heads, gq, max_blocks,
-                          nparts, q_stride, kv_fp8 != 0, window, stream);
+                          nparts, q_stride, kv_fp8 != 0, window, sink, stream);
   } else if (head_dim == 64) {
     launch_decode_gq<64>((bf16*)out, (float*)part_out, (const bf16*)q,
                          (const bf16*)k_cache, (const bf16*)v_cache,
                          (const int*)block_tables, (const int*)seq_lens, scale,
                          num_seqs, num_kv_heads, gq, max_blocks, nparts,
-                         q_stride, kv_fp8 != 0, window, stream);
+                         q_stride, kv_fp8 != 0, window, sink, stream);
   }
 }

@@ -57,9 +57,14 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
     const int* __restrict__ cu_seqlens_q,  // [num_seqs + 1]
     const int* __restrict__ tile_info,     // [ntiles, 2] = (seq_idx, q0)
     const float scale, const int num_q_heads, const int num_kv_heads,
-    const int max_blocks, const int64_t q_stride, const int window) {
+    const int max_blocks, const int64_t q_stride, const int window,
+    const int sink) {
   constexpr int CHUNKS = HEAD_DIM / 16;
   constexpr int STEPS = HEAD_DIM / 32;
+  // The XOR swizzle of K rows flips byte bits 4..6: it stays inside a row
+  // only when the row is a power of two of at least 128 bytes. Other head
+  // sizes (32, 96, ...) keep K rows unswizzled.
+  constexpr int SWZ = ((HEAD_DIM & (HEAD_DIM - 1)) == 0 && HEAD_DIM >= 64) ? 1 : 0;
 
   const int h = blockIdx.x;
   const int kvh = h / (num_q_heads / num_kv_heads);
@@ -101,8 +106,10 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
     }
   }
 
-  float m_run = -FLT_MAX;
-  float l_run = 0.f;
+  // sink: every softmax also holds a key of score 0 that has no value —
+  // the running state starts at (max 0, sum 1) instead of (-inf, 0)
+  float m_run = sink ? 0.f : -FLT_MAX;
+  float l_run = sink ? 1.f : 0.f;
   f32x4 oacc[CHUNKS];
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) oacc[c] = {0.f, 0.f, 0.f, 0.f};
@@ -153,7 +160,7 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
           }
         }
         const int row_byte = col8 * 2;
-        const int swz = row_byte ^ ((key & 7) << 4);
+        const int swz = row_byte ^ (SWZ * ((key & 7) << 4));
         *reinterpret_cast<ushort8*>(reinterpret_cast<char*>(&k_lds[key][0]) +
                                     swz) = kv;
         *reinterpret_cast<ushort8*>(
@@ -172,7 +179,7 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
 #pragma unroll
       for (int st = 0; st < STEPS; ++st) {
         const int col_byte = (st * 32 + ext_frag_k(la, 0)) * 2;
-        const int swz = col_byte ^ ((key & 7) << 4);
+        const int swz = col_byte ^ (SWZ * ((key & 7) << 4));
         ushort8 u = *reinterpret_cast<const ushort8*>(
             reinterpret_cast<const char*>(&k_lds[key][0]) + swz);
         sc[sub] =
@@ -285,35 +292,21 @@ extern "C" void arks_attn_extend_paged(
     const void* block_tables, const void* kv_lens, const void* cu_seqlens_q,
     const void* tile_info, int ntiles, float scale, int num_q_heads,
     int num_kv_heads, int head_dim, int max_blocks, int64_t q_stride,
-    int kv_fp8, int window, hipStream_t stream) {
+    int kv_fp8, int window, int sink, hipStream_t stream) {
   dim3 grid(num_q_heads, ntiles), block(256);
-  if (head_dim == 128 && kv_fp8) {
-    hipLaunchKernelGGL((attn_extend_kernel<128, true>), grid, block, 0, stream,
-                       (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
-                       (const bf16*)v_cache, (const int*)block_tables,
-                       (const int*)kv_lens, (const int*)cu_seqlens_q,
-                       (const int*)tile_info, scale, num_q_heads, num_kv_heads,
-                       max_blocks, q_stride, window);
-  } else if (head_dim == 64 && kv_fp8) {
-    hipLaunchKernelGGL((attn_extend_kernel<64, true>), grid, block, 0, stream,
-                       (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
-                       (const bf16*)v_cache, (const int*)block_tables,
-                       (const int*)kv_lens, (const int*)cu_seqlens_q,
-                       (const int*)tile_info, scale, num_q_heads, num_kv_heads,
-                       max_blocks, q_stride, window);
-  } else if (head_dim == 128) {
-    hipLaunchKernelGGL((attn_extend_kernel<128, false>), grid, block, 0, stream,
-                       (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
-                       (const bf16*)v_cache, (const int*)block_tables,
-                       (const int*)kv_lens, (const int*)cu_seqlens_q,
-                       (const int*)tile_info, scale, num_q_heads, num_kv_heads,
-                       max_blocks, q_stride, window);
-  } else if (head_dim == 64) {
-    hipLaunchKernelGGL((attn_extend_kernel<64, false>), grid, block, 0, stream,
-                       (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
-                       (const bf16*)v_cache, (const int*)block_tables,
-                       (const int*)kv_lens, (const int*)cu_seqlens_q,
-                       (const int*)tile_info, scale, num_q_heads, num_kv_heads,
-                       max_blocks, q_stride, window);
-  }
+#define ARKS_EXT(D, F8)                                                       \
+  hipLaunchKernelGGL((attn_extend_kernel<D, F8>), grid, block, 0, stream,     \
+                     (bf16*)out, (const bf16*)q, (const bf16*)k_cache,        \
+                     (const bf16*)v_cache, (const int*)block_tables,          \
+                     (const int*)kv_lens, (const int*)cu_seqlens_q,           \
+                     (const int*)tile_info, scale, num_q_heads, num_kv_heads, \
+                     max_blocks, q_stride, window, sink)
+  if (head_dim == 128 && kv_fp8) ARKS_EXT(128, true);
+  else if (head_dim == 64 && kv_fp8) ARKS_EXT(64, true);
+  else if (head_dim == 128) ARKS_EXT(128, false);
+  else if (head_dim == 64) ARKS_EXT(64, false);
+  else if (head_dim == 32) ARKS_EXT(32, false);
+  else if (head_dim == 96) ARKS_EXT(96, false);
+  else if (head_dim == 256) ARKS_EXT(256, false);
+#undef ARKS_EXT
 }

@@ -74,7 +74,8 @@ __global__ __launch_bounds__(512) void attn_extend2_kernel(
     const int* __restrict__ tile_info,
     float* __restrict__ part_ws,  // [ntiles, Hq, QTILE, D+2] f32 slabs
     const float scale, const int num_q_heads, const int num_kv_heads,
-    const int max_blocks, const int64_t q_stride, const int window) {
+    const int max_blocks, const int64_t q_stride, const int window,
+    const int sink) {
   constexpr int STEPS = HEAD_DIM / 16;   // QK^T K-contraction steps
   constexpr int DTILES = HEAD_DIM / 32;  // 32-dim output tiles
   constexpr int CB = HEAD_DIM / 16;      // 16-col blocks per key row
@@ -129,8 +130,11 @@ __global__ __launch_bounds__(512) void attn_extend2_kernel(
   // below any real score that exp2(fma(sentinel, scale2, -m*scale2))
   // underflows to 0 with no per-element select.
   constexpr float MASKED = -3e38f;
-  float m_run = -1e30f;
-  float l_run = 0.f;
+  // sink (a value-less key of score 0 in every softmax): the first KV part
+  // of a tile starts from (max 0, sum 1); the flash merge of split tiles
+  // then carries it like any other key
+  float m_run = (sink && part == 0) ? 0.f : -1e30f;
+  float l_run = (sink && part == 0) ? 1.f : 0.f;
   f32x16 oacc[DTILES];
 #pragma unroll
   for (int n = 0; n < DTILES; ++n) oacc[n] = {};
@@ -482,7 +486,7 @@ extern "C" void arks_attn_extend_paged2(
     const void* block_tables, const void* kv_lens, const void* cu_seqlens_q,
     const void* tile_info, void* part_ws, int ntiles, float scale,
     int num_q_heads, int num_kv_heads, int head_dim, int max_blocks,
-    int64_t q_stride, int window, hipStream_t stream) {
+    int64_t q_stride, int window, int sink, hipStream_t stream) {
   dim3 grid(num_q_heads, ntiles), block(512);
   static bool attr_set[2] = {false, false};
   auto launch = [&](auto kern, int lds_bytes, int idx) {
@@ -498,7 +502,7 @@ extern "C" void arks_attn_extend_paged2(
                        (const int*)kv_lens, (const int*)cu_seqlens_q,
                        (const int*)tile_info, (float*)part_ws, scale,
                        num_q_heads, num_kv_heads, max_blocks, q_stride,
-                       window);
+                       window, sink);
   };
   if (head_dim == 128) {
     constexpr int LDS = (2 * 64 * 128 + 2 * 16 * 8 * VBLK_ELEMS) * 2;

@@ -11,6 +11,8 @@
 
 namespace py = pybind11;
 
+#include "attn_bindings.h"
+
 // --- kernel launchers (see the .hip files) ---
 extern "C" {
 void arks_rmsnorm(void* out, const void* input, const void* weight, float eps,
@@ -40,38 +42,12 @@ void arks_rope_and_cache(const void* positions, void* q, void* k,
                          int num_tokens, int head_dim, int num_q_heads,
                          int num_kv_heads, int block_size, int64_t q_stride,
                          int64_t k_stride, int kv_fp8, hipStream_t stream);
-void arks_attn_decode_paged(void* out, void* part_out, const void* q,
-                            const void* k_cache, const void* v_cache,
-                            const void* block_tables, const void* seq_lens,
-                            float scale, int num_seqs, int num_q_heads,
-                            int num_kv_heads, int head_dim, int max_blocks,
-                            int nparts, int64_t q_stride, int kv_fp8,
-                            int window, hipStream_t stream);
 void arks_attn_prefill_varlen(void* out, const void* q, const void* k,
                               const void* v, const void* cu_seqlens,
                               const void* tile_info, int ntiles, float scale,
                               int num_q_heads, int num_kv_heads, int head_dim,
                               int64_t q_stride, int64_t kv_stride, int window,
                               hipStream_t stream);
-void arks_attn_extend_paged(void* out, const void* q, const void* k_cache,
-                            const void* v_cache, const void* block_tables,
-                            const void* kv_lens, const void* cu_seqlens_q,
-                            const void* tile_info, int ntiles, float scale,
-                            int num_q_heads, int num_kv_heads, int head_dim,
-                            int max_blocks, int64_t q_stride, int kv_fp8,
-                            int window, hipStream_t stream);
-void arks_attn_extend_paged2(void* out, const void* q, const void* k_cache,
-                             const void* v_cache, const void* block_tables,
-                             const void* kv_lens, const void* cu_seqlens_q,
-                             const void* tile_info, void* part_ws, int ntiles,
-                             float scale, int num_q_heads, int num_kv_heads,
-                             int head_dim, int max_blocks, int64_t q_stride,
-                             int window, hipStream_t stream);
-void arks_attn_extend2_combine(void* out, const void* part_ws,
-                               const void* combine_table,
-                               const void* cu_seqlens_q, int n_split,
-                               float scale, int num_q_heads, int head_dim,
-                               hipStream_t stream);
 void arks_quant_fp8_rows(void* out, void* inv_scale, const void* x, int rows,
                          int cols, hipStream_t stream);
 void arks_rmsnorm_fp8(void* out, void* inv_scale, const void* input,
@@ -116,30 +92,10 @@ hipStream_t current_stream() {
 }
 
 // KV caches may be bf16 or fp8 e4m3 (kv_cache_dtype="fp8"); returns fp8?
-bool check_kv_cache(const torch::Tensor& t, const char* name) {
-  TORCH_CHECK(t.is_cuda(), name, " must be on GPU");
-  TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
-  if (t.scalar_type() == torch::kFloat8_e4m3fn) return true;
-  TORCH_CHECK(t.scalar_type() == torch::kBFloat16, name, " must be bf16/fp8");
-  return false;
-}
 
-void check_bf16_contig(const torch::Tensor& t, const char* name) {
-  TORCH_CHECK(t.is_cuda(), name, " must be on GPU");
-  TORCH_CHECK(t.scalar_type() == torch::kBFloat16, name, " must be bf16");
-  TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
-}
 
 // bf16 tensor whose trailing dims are contiguous; dim-0 rows may be strided
 // (a view into the fused QKV buffer).
-void check_bf16_rowstrided(const torch::Tensor& t, const char* name) {
-  TORCH_CHECK(t.is_cuda(), name, " must be on GPU");
-  TORCH_CHECK(t.scalar_type() == torch::kBFloat16, name, " must be bf16");
-  TORCH_CHECK(t.stride(-1) == 1, name, " last dim must be contiguous");
-  if (t.dim() == 3) {
-    TORCH_CHECK(t.stride(1) == t.size(2), name, " inner dims must be dense");
-  }
-}
 
 void rmsnorm(torch::Tensor out, torch::Tensor input, torch::Tensor weight,
              double eps) {
@@ -238,42 +194,6 @@ void rope_and_cache(torch::Tensor positions, torch::Tensor q,
                       k.stride(0), kv_fp8 ? 1 : 0, current_stream());
 }
 
-void attention_decode_paged(torch::Tensor out, torch::Tensor q,
-                            torch::Tensor k_cache, torch::Tensor v_cache,
-                            torch::Tensor block_tables, torch::Tensor seq_lens,
-                            double scale, torch::Tensor part_out,
-                            int64_t nparts, int64_t window) {
-  check_bf16_contig(out, "out");
-  check_bf16_rowstrided(q, "q");
-  const bool kv_fp8 = check_kv_cache(k_cache, "k_cache");
-  check_kv_cache(v_cache, "v_cache");
-  TORCH_CHECK(block_tables.scalar_type() == torch::kInt32);
-  TORCH_CHECK(seq_lens.scalar_type() == torch::kInt32);
-  const int num_seqs = q.size(0);
-  const int num_q_heads = q.size(1);
-  const int head_dim = q.size(2);
-  const int num_kv_heads = k_cache.size(1);
-  TORCH_CHECK(k_cache.size(2) == 16, "KV block size must be 16");
-  TORCH_CHECK(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128");
-  const int gq = num_q_heads / num_kv_heads;
-  TORCH_CHECK(gq >= 1 && gq <= 8 && gq * num_kv_heads == num_q_heads,
-              "q/kv head ratio must be integral and <= 8");
-  const int max_blocks = block_tables.size(1);
-  if (nparts > 1) {
-    TORCH_CHECK(part_out.scalar_type() == torch::kFloat32 &&
-                part_out.numel() >=
-                    (int64_t)num_seqs * num_kv_heads * nparts * gq *
-                        (head_dim + 2),
-                "part_out workspace too small");
-  }
-  arks_attn_decode_paged(out.data_ptr(),
-                         nparts > 1 ? part_out.data_ptr() : nullptr,
-                         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                         block_tables.data_ptr(), seq_lens.data_ptr(),
-                         (float)scale, num_seqs, num_q_heads, num_kv_heads,
-                         head_dim, max_blocks, (int)nparts, q.stride(0),
-                         kv_fp8 ? 1 : 0, (int)window, current_stream());
-}
 
 void attention_prefill_varlen(torch::Tensor out, torch::Tensor q,
                               torch::Tensor k, torch::Tensor v,
@@ -299,88 +219,9 @@ void attention_prefill_varlen(torch::Tensor out, torch::Tensor q,
                            k.stride(0), (int)window, current_stream());
 }
 
-void attention_extend_paged(torch::Tensor out, torch::Tensor q,
-                            torch::Tensor k_cache, torch::Tensor v_cache,
-                            torch::Tensor block_tables, torch::Tensor kv_lens,
-                            torch::Tensor cu_seqlens_q, torch::Tensor tile_info,
-                            double scale, int64_t window) {
-  check_bf16_contig(out, "out");
-  check_bf16_rowstrided(q, "q");
-  const bool kv_fp8 = check_kv_cache(k_cache, "k_cache");
-  check_kv_cache(v_cache, "v_cache");
-  TORCH_CHECK(block_tables.scalar_type() == torch::kInt32);
-  TORCH_CHECK(kv_lens.scalar_type() == torch::kInt32);
-  TORCH_CHECK(cu_seqlens_q.scalar_type() == torch::kInt32);
-  TORCH_CHECK(tile_info.scalar_type() == torch::kInt32);
-  TORCH_CHECK(tile_info.dim() == 2 && tile_info.size(1) == 2);
-  const int num_q_heads = q.size(1);
-  const int head_dim = q.size(2);
-  const int num_kv_heads = k_cache.size(1);
-  TORCH_CHECK(k_cache.size(2) == 16, "KV block size must be 16");
-  TORCH_CHECK(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128");
-  const int ntiles = tile_info.size(0);
-  const int max_blocks = block_tables.size(1);
-  arks_attn_extend_paged(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
-                         v_cache.data_ptr(), block_tables.data_ptr(),
-                         kv_lens.data_ptr(), cu_seqlens_q.data_ptr(),
-                         tile_info.data_ptr(), ntiles, (float)scale,
-                         num_q_heads, num_kv_heads, head_dim, max_blocks,
-                         q.stride(0), kv_fp8 ? 1 : 0, (int)window,
-                         current_stream());
-}
 
 // 8-wave 32x32-MFMA ladder (attn_extend2.hip): 256-row q tiles, bf16 KV.
-void attention_extend_paged2(torch::Tensor out, torch::Tensor q,
-                             torch::Tensor k_cache, torch::Tensor v_cache,
-                             torch::Tensor block_tables, torch::Tensor kv_lens,
-                             torch::Tensor cu_seqlens_q,
-                             torch::Tensor tile_info, torch::Tensor part_ws,
-                             double scale, int64_t window) {
-  check_bf16_contig(out, "out");
-  check_bf16_rowstrided(q, "q");
-  check_bf16_contig(k_cache, "k_cache");
-  check_bf16_contig(v_cache, "v_cache");
-  TORCH_CHECK(block_tables.scalar_type() == torch::kInt32);
-  TORCH_CHECK(kv_lens.scalar_type() == torch::kInt32);
-  TORCH_CHECK(cu_seqlens_q.scalar_type() == torch::kInt32);
-  TORCH_CHECK(tile_info.scalar_type() == torch::kInt32);
-  TORCH_CHECK(tile_info.dim() == 2 && tile_info.size(1) == 4,
-              "tile_info rows are (seq, q0, part, nparts)");
-  const int num_q_heads = q.size(1);
-  const int head_dim = q.size(2);
-  const int num_kv_heads = k_cache.size(1);
-  TORCH_CHECK(k_cache.size(2) == 16, "KV block size must be 16");
-  TORCH_CHECK(head_dim == 64 || head_dim == 128, "head_dim must be 64 or 128");
-  const int ntiles = tile_info.size(0);
-  const int max_blocks = block_tables.size(1);
-  void* ws = nullptr;
-  if (part_ws.numel() > 0) {
-    // sized by the host: split rows sort first, so only their slabs exist
-    TORCH_CHECK(part_ws.scalar_type() == torch::kFloat32);
-    ws = part_ws.data_ptr();
-  }
-  arks_attn_extend_paged2(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
-                          v_cache.data_ptr(), block_tables.data_ptr(),
-                          kv_lens.data_ptr(), cu_seqlens_q.data_ptr(),
-                          tile_info.data_ptr(), ws, ntiles, (float)scale,
-                          num_q_heads, num_kv_heads, head_dim, max_blocks,
-                          q.stride(0), (int)window, current_stream());
-}
 
-void attention_extend2_combine(torch::Tensor out, torch::Tensor part_ws,
-                               torch::Tensor combine_table,
-                               torch::Tensor cu_seqlens_q, double scale) {
-  check_bf16_rowstrided(out, "out");
-  TORCH_CHECK(part_ws.scalar_type() == torch::kFloat32);
-  TORCH_CHECK(combine_table.scalar_type() == torch::kInt32 &&
-              combine_table.dim() == 2 && combine_table.size(1) == 4);
-  const int num_q_heads = out.size(1);
-  const int head_dim = out.size(2);
-  arks_attn_extend2_combine(out.data_ptr(), part_ws.data_ptr(),
-                            combine_table.data_ptr(), cu_seqlens_q.data_ptr(),
-                            combine_table.size(0), (float)scale, num_q_heads,
-                            head_dim, current_stream());
-}
 
 void skinny_gemm(torch::Tensor out, torch::Tensor part, torch::Tensor a,
                  torch::Tensor w, c10::optional<torch::Tensor> bias,
@@ -653,17 +494,14 @@ void mfma_probe(torch::Tensor d, torch::Tensor a, torch::Tensor b) {
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  def_paged_attention(m);
   m.def("rmsnorm", &rmsnorm);
   m.def("fused_add_rmsnorm", &fused_add_rmsnorm);
   m.def("silu_mul", &silu_mul);
   m.def("rope_inplace", &rope_inplace);
   m.def("reshape_and_cache", &reshape_and_cache);
   m.def("rope_and_cache", &rope_and_cache);
-  m.def("attention_decode_paged", &attention_decode_paged);
   m.def("attention_prefill_varlen", &attention_prefill_varlen);
-  m.def("attention_extend_paged", &attention_extend_paged);
-  m.def("attention_extend_paged2", &attention_extend_paged2);
-  m.def("attention_extend2_combine", &attention_extend2_combine);
   m.def("quant_fp8_rows", &quant_fp8_rows);
   m.def("rmsnorm_fp8", &rmsnorm_fp8);
   m.def("silu_mul_fp8", &silu_mul_fp8);

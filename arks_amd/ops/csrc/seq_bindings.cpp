@@ -5,6 +5,8 @@
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime.h>
 
+#include "attn_bindings.h"
+
 extern "C" {
 void arks_seq_token_shift(void* xs, void* xa, const void* x, const void* w,
                           void* state, const void* cu, const void* seq_lens,
@@ -26,6 +28,9 @@ void arks_seq_qk_norm_rope_cache(
     int n_vrot, void* k_cache, void* v_cache, const void* slot_mapping, int T,
     int H, int G, int D, int V, int block_size, int interleaved, int act_f32,
     hipStream_t stream);
+void arks_seq_unrotate_rows(void* out, const void* positions, const void* freq,
+                            int T, int H, int V, int interleaved, int act_f32,
+                            hipStream_t stream);
 int arks_seq_attn_sink_generic(
     void* out, const void* q, const void* k_cache, const void* v_cache,
     const void* block_tables, const void* seq_lens, const void* cu,
@@ -301,6 +306,20 @@ void attention_sink_paged(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
               D, ", ", V, ")");
 }
 
+void unrotate_rows(Tensor out, Tensor positions, Tensor freq_v,
+                   bool interleaved) {
+  const int f32 = act_flag(out, "out");
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 3);
+  check_i64(positions, "positions");
+  check_f32(freq_v, "inv_freq_v");
+  TORCH_CHECK(positions.numel() == out.size(0) &&
+              2 * freq_v.numel() == out.size(2));
+  arks_seq_unrotate_rows(out.data_ptr(), positions.data_ptr(),
+                         freq_v.data_ptr(), out.size(0), out.size(1),
+                         out.size(2), interleaved ? 1 : 0, f32,
+                         current_stream());
+}
+
 void lightning_scan(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
                     Tensor state, Tensor cu, Tensor seq_lens, Tensor slots,
                     int64_t max_q_len) {
@@ -389,6 +408,8 @@ void selective_scan(Tensor out, Tensor u, Tensor dbc, Tensor z, Tensor dt_w,
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  def_paged_attention(m);
+  m.def("unrotate_rows", &unrotate_rows);
   m.def("token_shift", &token_shift);
   m.def("gated_norm_residual", &gated_norm_residual);
   m.def("rms_norm_f32", &rms_norm_f32);

@@ -168,9 +168,41 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
   }
 }
 
+// Turn every head row of out [T, H, V] back by its row's position: pair m
+// by -pos * freq[m] (the cache holds values turned forward by their own
+// positions, so the weighted sum comes out in the query's frame).
+template <typename AT>
+__global__ __launch_bounds__(64) void unrotate_rows_kernel(
+    AT* __restrict__ out, const int64_t* __restrict__ positions,
+    const float* __restrict__ freq, int V, int interleaved) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  AT* row = out + ((int64_t)t * gridDim.y + h) * V;
+  const float pos = (float)positions[t];
+  const int npairs = V / 2;
+  for (int i = threadIdx.x; i < npairs; i += 64) {
+    const int d0 = interleaved ? 2 * i : i;
+    const int d1 = interleaved ? 2 * i + 1 : i + npairs;
+    const float a = Act<AT>::ld(row + d0), b = Act<AT>::ld(row + d1);
+    float sn, cs;
+    sincosf(-pos * freq[i], &sn, &cs);
+    Act<AT>::st(row + d0, a * cs - b * sn);
+    Act<AT>::st(row + d1, b * cs + a * sn);
+  }
+}
+
 }  // namespace arks
 
 using namespace arks;
+
+extern "C" void arks_seq_unrotate_rows(void* out, const void* positions,
+                                       const void* freq, int T, int H, int V,
+                                       int interleaved, int act_f32,
+                                       hipStream_t stream) {
+  if (T == 0) return;
+  SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
+      (unrotate_rows_kernel<AT>), dim3(T, H), dim3(64), 0, stream, (AT*)out,
+      (const int64_t*)positions, (const float*)freq, V, interleaved));
+}
 
 extern "C" void arks_seq_token_shift(void* xs, void* xa, const void* x,
                                      const void* w, void* state, const void* cu,

@@ -50,6 +50,12 @@ def parse_args():
     # checkpoint to disk once, drop the page cache, and time disk -> HBM
     # through the pinned double-buffer loader (not the synthetic
     # random-init path the serving bench uses).
+    # NOT the headline either: prefill and decode throughput of a layer-list
+    # design (Gagorax) at real layer sizes beside the closest llama-family
+    # model cut to the same width and depth, one JSON line per model and
+    # phase. --design-only NAME runs one of the two (profiling).
+    p.add_argument("--design-bench", action="store_true")
+    p.add_argument("--design-only", choices=["gagorax", "llama"], default=None)
     p.add_argument("--cold-start", action="store_true")
     p.add_argument("--ckpt-dir", default="/tmp/arks_ckpt")
     return p.parse_args()
@@ -114,10 +120,92 @@ def run_cold_start(args):
     print(json.dumps(result))
 
 
+def run_design_bench(args):
+    """Gagorax (8 blocks at the sizes of an 8B model) against llama-3-8b cut
+    to 8 layers: prefill tokens/s for one long prompt and for a batch of
+    prompts, decode tokens/s for a batch at a fixed context. Random weights,
+    synthetic tokens, one GPU."""
+    import dataclasses
+
+    from arks_amd.config import EngineConfig, PRESET_CONFIGS
+    from arks_amd.engine import LLMEngine, SamplingParams
+
+    PRESET_CONFIGS["llama-3-8b-8l"] = dataclasses.replace(
+        PRESET_CONFIGS["llama-3-8b"], num_hidden_layers=8)
+    use_gpu = torch.cuda.is_available()
+    models = {"gagorax": "gagorax-8b-slice", "llama": "llama-3-8b-8l"}
+    prefills = [(1, 8192), (8, 2048), (32, 128)]  # (prompts, tokens each)
+    dec_batch, dec_ctx = args.batch, args.input_len
+    for key, preset in models.items():
+        if args.design_only and key != args.design_only:
+            continue
+        blocks = max(dec_batch * (dec_ctx + args.steps + args.warmup + 64),
+                     max(b * n for b, n in prefills) + 1024) // 16 + 64
+        cfg = EngineConfig(
+            preset=preset, device="cuda" if use_gpu else "cpu",
+            max_num_seqs=max(dec_batch, 64), max_num_batched_tokens=16384,
+            max_model_len=16384, kv_cache_blocks=blocks, seed=args.seed,
+            enable_prefix_caching=False)
+        engine = LLMEngine(cfg)
+        vocab = engine.model_cfg.vocab_size
+        g = torch.Generator().manual_seed(args.seed)
+
+        def prompts(b, n):
+            return [torch.randint(0, vocab - 1, (n,), generator=g).tolist()
+                    for _ in range(b)]
+
+        def sync():
+            if use_gpu:
+                torch.cuda.synchronize()
+
+        engine.generate(prompts(2, 40), SamplingParams(max_tokens=3, ignore_eos=True))
+        for b, n in prefills:
+            best = None
+            for rep in range(3):  # first repetition warms shapes up
+                for pr in prompts(b, n):
+                    engine.add_request(pr, SamplingParams(max_tokens=1, ignore_eos=True))
+                sync()
+                t0 = time.time()
+                while engine.has_work():
+                    engine.step()
+                sync()
+                dt = time.time() - t0
+                best = dt if best is None or rep and dt < best else best
+            print(json.dumps({
+                "metric": "prefill_tok_s", "model": preset, "value": round(b * n / best, 1),
+                "unit": "tok/s", "prompts": b, "prompt_len": n,
+                "ms": round(best * 1000, 2), "dtype": "bf16", "data": "synthetic"}), flush=True)
+        sp = SamplingParams(max_tokens=args.warmup + args.steps + 8, ignore_eos=True)
+        for pr in prompts(dec_batch, dec_ctx):
+            engine.add_request(pr, sp)
+        while engine.scheduler.num_waiting > 0:
+            engine.step()
+        for _ in range(args.warmup):
+            engine.step()
+        sync()
+        t0 = time.time()
+        n_out = 0
+        for _ in range(args.steps):
+            n_out += len(engine.step())
+        sync()
+        dt = time.time() - t0
+        print(json.dumps({
+            "metric": "decode_tok_s", "model": preset, "value": round(n_out / dt, 1),
+            "unit": "tok/s", "batch": dec_batch, "context": dec_ctx,
+            "ms_per_step": round(dt / args.steps * 1000, 3), "dtype": "bf16",
+            "data": "synthetic"}), flush=True)
+        del engine
+        if use_gpu:
+            torch.cuda.empty_cache()
+
+
 def main():
     args = parse_args()
     if args.cold_start:
         run_cold_start(args)
+        return
+    if args.design_bench:
+        run_design_bench(args)
         return
     rank = int(os.environ.get("RANK", 0))
     world = int(os.environ.get("WORLD_SIZE", 1))

@@ -245,3 +245,26 @@ def test_greedy_generation_through_the_scheduler(tmp_path, device, dtype):
                     1e-3 if dtype == "float32" else 0.15), (top2, got_tok)
             cur = got_tok  # follow the engine's choice
     assert eng.scheduler.allocator.num_free == eng.runner.num_blocks
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("dim,heads,kv", [(32, 4, 2), (64, 8, 1), (96, 2, 2), (128, 4, 2)])
+def test_attention_head_sizes_of_the_mfma_kernels(tmp_path, device, dtype, dim, heads, kv):
+    """Equal q/k and value sizes the matrix-core kernels are built for: a
+    long prompt (the 256-row kernel where it exists), short portions (the
+    64-row kernel), single tokens (flash decode) and mixes of them."""
+    cfg = model_cfg([attn(heads=heads, kv=kv, dim=dim, vdim=dim, rot=dim // 2, mlp=FF),
+                     attn(heads=heads, kv=kv, dim=dim, vdim=dim)], width=64)
+    w = write_checkpoint(tmp_path / "m", cfg, seed=dim)
+    ta, tb = toks(330, seed=4), toks(40, seed=6)
+    orc = Oracle(cfg, w)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=512)
+    steps = [[("a", ta[:300], False)],
+             [("a", ta[300:301], False), ("b", tb[:30], False)],
+             [("a", ta[301:302], False), ("b", tb[30:31], False)],
+             [("a", ta[302:303], False), ("b", tb[31:32], False)],
+             [("a", ta[303:330], True), ("b", tb[32:33], False)],
+             [("b", tb[33:], True)]]
+    got = replay(eng, tmp_path, steps)
+    assert rel_err(got["a"], orc.run(ta)) < TOL[dtype]
+    assert rel_err(got["b"], orc.run(tb)) < TOL[dtype]
