@@ -42,6 +42,35 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return F.linear(x, w)
 
 
+_MM_OUT_DTYPE = [True]  # torch.mm(..., out_dtype=) available
+
+
+def linear_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """x @ w^T with fp32 OUTPUT from rows of the model's dtype (bf16 inputs,
+    fp32 accumulate, no rounding of the result)."""
+    if x.dtype == torch.float32:
+        return F.linear(x, w)
+    if _MM_OUT_DTYPE[0]:
+        try:
+            return torch.mm(x, w.t(), out_dtype=torch.float32)
+        except (TypeError, RuntimeError):
+            _MM_OUT_DTYPE[0] = False
+    return F.linear(x, w).float()
+
+
+def step_chunks(batch: ForwardBatch, device):
+    """Chunk metadata of this step for the chunk-parallel recurrent prefill
+    (None for steps whose rows per sequence all fit one chunk, and inside
+    captured decode graphs)."""
+    if (device.type != "cuda" or batch.seq_lens_list is None
+            or batch.max_q_len <= ops.SCAN_CHUNK):
+        return None
+    if "scan_chunks" not in batch.tile_cache:
+        batch.tile_cache["scan_chunks"] = ops.scan_chunks(
+            batch.seq_lens_list, device)
+    return batch.tile_cache["scan_chunks"]
+
+
 def _param(*shape, dtype):
     return nn.Parameter(torch.zeros(*shape, dtype=dtype), requires_grad=False)
 
@@ -155,7 +184,8 @@ class LightningMixer(nn.Module):
         g = p[:, 2 * H * D + H * V:]
         o = ops.lightning_scan(q, k, v, self.decay, cache["S"],
                                batch.cu_seqlens, batch.seq_lens,
-                               batch.state_slots, batch.max_q_len)
+                               batch.state_slots, batch.max_q_len,
+                               step_chunks(batch, xs.device))
         y = ops.gated_rmsnorm(o.view(T, H * V), self.norm, g, self.eps, xs.dtype)
         return linear(y, self.o)
 
@@ -177,6 +207,10 @@ class Mamba1Mixer(nn.Module):
         self.D = _param(inner, dtype=f32)
         self.register_buffer("A", torch.zeros(inner, state, dtype=f32),
                              persistent=False)
+        # dt's projection as a GEMM operand (the kernels can also project
+        # in place from the fp32 dt_w: tiny ranks, CPU reference)
+        self.register_buffer("dt_w_mm", torch.zeros(inner, dt_rank, dtype=dtype),
+                             persistent=False)
 
     def weight_map(self) -> dict:
         return {"in": (self.w_in, 0), "x": (self.w_x, 0), "o": (self.o, 0),
@@ -186,6 +220,7 @@ class Mamba1Mixer(nn.Module):
 
     def finish_loading(self) -> None:
         self.A.copy_(-torch.exp(self.A_log.data.float()))
+        self.dt_w_mm.copy_(self.dt_w.data)
 
     def cache_layout(self, block_size: int, dtype) -> dict:
         out = {"ssm": ("slot", (self.C, self.N), torch.float32)}
@@ -201,10 +236,13 @@ class Mamba1Mixer(nn.Module):
             batch.cu_seqlens, batch.seq_lens, batch.state_slots,
             batch.token_seq)
         dbc = linear(u, self.w_x)
+        dt_pre = None
+        if xs.is_cuda and self.R >= 8:
+            dt_pre = linear_f32(dbc[:, :self.R], self.dt_w_mm)
         y = ops.selective_scan(
             u, dbc, xz[:, C:], self.dt_w, self.dt_b, self.A, self.D,
             cache["ssm"], batch.cu_seqlens, batch.seq_lens, batch.state_slots,
-            batch.max_q_len)
+            batch.max_q_len, dt_pre, step_chunks(batch, xs.device))
         return linear(y, self.o)
 
 

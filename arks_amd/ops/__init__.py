@@ -709,14 +709,52 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
                                     inv_freq_v, interleaved)
 
 
+SCAN_CHUNK = 64  # rows per chunk of the chunk-parallel recurrent prefill
+
+
+def scan_chunks(q_lens: list[int], device, chunk: int = SCAN_CHUNK) -> dict:
+    """Cut every sequence's rows of this step into chunks of <= `chunk`
+    rows, as metadata of 'virtual sequences' the scan kernels can run in
+    parallel: pass 1 scans each chunk from zero state into a scratch slot
+    of its own (lens0: chunk starts at position 0), a small combine kernel
+    walks each sequence's chunks in order and leaves every chunk's START
+    state in its scratch slot, pass 2 scans again from those (lens1: start
+    > 0) and writes the outputs. Same arithmetic as the row-by-row scan up
+    to fp32 summation order."""
+    rows, off = [], [0]
+    for n in q_lens:
+        rows += [min(chunk, n - j) for j in range(0, n, chunk)]
+        off.append(len(rows))
+    t = lambda x: torch.tensor(x, dtype=torch.int32, device=device)
+    cu = [0]
+    for r in rows:
+        cu.append(cu[-1] + r)
+    return {"n": len(rows), "cu": t(cu), "lens0": t(rows),
+            "lens1": t([r + 1 for r in rows]), "rows": t(rows),
+            "slots": t(list(range(len(rows)))), "off": t(off)}
+
+
 def lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
-                   max_q_len=0):
+                   max_q_len=0, chunks=None):
+    """chunks (scan_chunks of this step): run the prefill chunk-parallel."""
     if q.is_cuda:
-        T, H, _ = q.shape
+        T, H, D = q.shape
         V = v.shape[2]
+        S = _native_seq()
         out = torch.empty((T, H, V), dtype=torch.float32, device=q.device)
-        _native_seq().lightning_scan(out, q, k, v, decay, state, cu_seqlens,
-                                     seq_lens, state_slots, max_q_len)
+        if chunks is not None and max_q_len > SCAN_CHUNK:
+            c = chunks
+            part = torch.empty((c["n"], H, D, V), dtype=torch.float32,
+                               device=q.device)
+            S.lightning_scan(out, q, k, v, decay, part, c["cu"], c["lens0"],
+                             c["slots"], SCAN_CHUNK)
+            S.lightning_combine(part, decay, state, c["off"], c["rows"],
+                                cu_seqlens, seq_lens, state_slots)
+            S.lightning_scan(out, q, k, v, decay, part, c["cu"], c["lens1"],
+                             c["slots"], SCAN_CHUNK)
+            return out
+        S.lightning_scan(out, q, k, v, decay, state, cu_seqlens, seq_lens,
+                         state_slots, max_q_len)
         return out
     return ref.lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens,
                               state_slots)
@@ -742,12 +780,28 @@ def causal_conv_silu(x, weight, bias, state, cu_seqlens, seq_lens,
 
 
 def selective_scan(u, dbc, z, dt_w, dt_b, A, Dp, state, cu_seqlens, seq_lens,
-                   state_slots, max_q_len=0):
+                   state_slots, max_q_len=0, dt_pre=None, chunks=None):
+    """dt_pre: fp32 [T, C] = dt_raw @ dt_w^T from a GEMM (else projected in
+    the kernel); chunks (scan_chunks of this step): chunk-parallel prefill."""
     if u.is_cuda:
+        S = _native_seq()
         out = torch.empty(u.shape, dtype=u.dtype, device=u.device)
-        _native_seq().selective_scan(out, u, dbc, z, dt_w, dt_b, A, Dp, state,
-                                     cu_seqlens, seq_lens, state_slots,
-                                     max_q_len)
+        if chunks is not None and max_q_len > SCAN_CHUNK:
+            c = chunks
+            C, N = A.shape
+            part = torch.empty((c["n"], C, N), dtype=torch.float32,
+                               device=u.device)
+            dsum = torch.empty((c["n"], C), dtype=torch.float32,
+                               device=u.device)
+            S.selective_scan(out, u, dbc, z, dt_w, dt_b, A, Dp, part, c["cu"],
+                             c["lens0"], c["slots"], dt_pre, dsum)
+            S.scan_combine(part, dsum, A, state, c["off"], cu_seqlens,
+                           seq_lens, state_slots)
+            S.selective_scan(out, u, dbc, z, dt_w, dt_b, A, Dp, part, c["cu"],
+                             c["lens1"], c["slots"], dt_pre, None)
+            return out
+        S.selective_scan(out, u, dbc, z, dt_w, dt_b, A, Dp, state, cu_seqlens,
+                         seq_lens, state_slots, dt_pre, None)
         return out
     return ref.selective_scan(u, dbc, z, dt_w, dt_b, A, Dp, state, cu_seqlens,
                               seq_lens, state_slots)

@@ -54,8 +54,17 @@ int arks_seq_selective_scan(void* out, const void* u, const void* dbc,
                             const void* dt_w, const void* dt_b, const void* A,
                             const void* Dp, void* state, const void* cu,
                             const void* seq_lens, const void* slots, int S,
-                            int C, int N, int R, int act_f32,
-                            hipStream_t stream);
+                            int C, int N, int R, const void* dt_pre,
+                            void* dsum, int act_f32, hipStream_t stream);
+void arks_seq_scan_combine(void* part, const void* dsum, const void* A,
+                           void* state, const void* chunk_off, const void* cu,
+                           const void* seq_lens, const void* slots, int S,
+                           int C, int N, hipStream_t stream);
+void arks_seq_lightning_combine(void* part, const void* decay, void* state,
+                                const void* chunk_off, const void* chunk_rows,
+                                const void* cu, const void* seq_lens,
+                                const void* slots, int S, int H, int DV,
+                                hipStream_t stream);
 }
 
 namespace {
@@ -375,7 +384,8 @@ void causal_conv_silu(Tensor out, Tensor x, Tensor w, Tensor bias,
 
 void selective_scan(Tensor out, Tensor u, Tensor dbc, Tensor z, Tensor dt_w,
                     Tensor dt_b, Tensor A, Tensor Dp, Tensor state, Tensor cu,
-                    Tensor seq_lens, Tensor slots, int64_t max_q_len) {
+                    Tensor seq_lens, Tensor slots, OptTensor dt_pre,
+                    OptTensor dsum) {
   const int f32 = act_flag(u, "u");
   const int T = u.size(0), C = u.size(1);
   TORCH_CHECK(u.is_contiguous() && out.is_contiguous() &&
@@ -396,13 +406,70 @@ void selective_scan(Tensor out, Tensor u, Tensor dbc, Tensor z, Tensor dt_w,
   TORCH_CHECK(state.dim() == 3 && state.size(1) == C && state.size(2) == N,
               "ssm state must be [slots, C, N]");
   const SeqMeta m = check_meta(cu, seq_lens, &slots, nullptr, T);
+  const void* dtp_p = nullptr;
+  void* dsum_p = nullptr;
+  if (dt_pre.has_value()) {
+    check_f32(*dt_pre, "dt_pre");
+    TORCH_CHECK(dt_pre->dim() == 2 && dt_pre->size(0) == T &&
+                dt_pre->size(1) == C, "dt_pre must be [T, C]");
+    dtp_p = dt_pre->data_ptr();
+  }
+  if (dsum.has_value()) {
+    check_f32(*dsum, "dsum");
+    TORCH_CHECK(dsum->numel() == (int64_t)m.S * C, "dsum must be [S, C]");
+    dsum_p = dsum->data_ptr();
+  }
   const int rc = arks_seq_selective_scan(
       out.data_ptr(), u.data_ptr(), dbc.data_ptr(), row_stride(dbc, "dbc"),
       z.data_ptr(), row_stride(z, "z"), dt_w.data_ptr(), dt_b.data_ptr(),
       A.data_ptr(), Dp.data_ptr(), state.data_ptr(), cu.data_ptr(),
-      seq_lens.data_ptr(), slots.data_ptr(), m.S, C, N, R, f32,
+      seq_lens.data_ptr(), slots.data_ptr(), m.S, C, N, R, dtp_p, dsum_p, f32,
       current_stream());
   TORCH_CHECK(rc == 0, "ssm state size beyond the kernel's limit (", N, ")");
+}
+
+// part [chunks, C, N], dsum [chunks, C]; chunk_off [S + 1] = each real
+// sequence's range of chunks
+void scan_combine(Tensor part, Tensor dsum, Tensor A, Tensor state,
+                  Tensor chunk_off, Tensor cu, Tensor seq_lens, Tensor slots) {
+  check_f32(part, "part");
+  check_f32(dsum, "dsum");
+  check_f32(A, "A");
+  check_f32(state, "ssm state");
+  const int C = A.size(0), N = A.size(1);
+  TORCH_CHECK(part.dim() == 3 && part.size(1) == C && part.size(2) == N &&
+              dsum.dim() == 2 && dsum.size(0) == part.size(0) &&
+              dsum.size(1) == C && state.size(1) == C && state.size(2) == N);
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, nullptr, 0);
+  check_i32(chunk_off, "chunk_off");
+  TORCH_CHECK(chunk_off.numel() == m.S + 1);
+  arks_seq_scan_combine(part.data_ptr(), dsum.data_ptr(), A.data_ptr(),
+                        state.data_ptr(), chunk_off.data_ptr(), cu.data_ptr(),
+                        seq_lens.data_ptr(), slots.data_ptr(), m.S, C, N,
+                        current_stream());
+}
+
+void lightning_combine(Tensor part, Tensor decay, Tensor state,
+                       Tensor chunk_off, Tensor chunk_rows, Tensor cu,
+                       Tensor seq_lens, Tensor slots) {
+  check_f32(part, "part");
+  check_f32(decay, "decay");
+  check_f32(state, "state");
+  TORCH_CHECK(part.dim() == 4 && state.dim() == 4 &&
+              part.size(1) == state.size(1) && part.size(2) == state.size(2) &&
+              part.size(3) == state.size(3));
+  const int H = state.size(1), DV = state.size(2) * state.size(3);
+  TORCH_CHECK(decay.numel() == H);
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, nullptr, 0);
+  check_i32(chunk_off, "chunk_off");
+  check_i32(chunk_rows, "chunk_rows");
+  TORCH_CHECK(chunk_off.numel() == m.S + 1 &&
+              chunk_rows.numel() == part.size(0));
+  arks_seq_lightning_combine(part.data_ptr(), decay.data_ptr(),
+                             state.data_ptr(), chunk_off.data_ptr(),
+                             chunk_rows.data_ptr(), cu.data_ptr(),
+                             seq_lens.data_ptr(), slots.data_ptr(), m.S, H, DV,
+                             current_stream());
 }
 
 }  // namespace
@@ -420,4 +487,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("lightning_scan", &lightning_scan);
   m.def("causal_conv_silu", &causal_conv_silu);
   m.def("selective_scan", &selective_scan);
+  m.def("scan_combine", &scan_combine);
+  m.def("lightning_combine", &lightning_combine);
 }

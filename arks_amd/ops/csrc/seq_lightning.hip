@@ -60,9 +60,53 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(
   }
 }
 
+// Chunk-parallel prefill, middle step (see scan_combine_kernel in
+// seq_mamba.hip): part[k] = end state of chunk k scanned from zero; replace
+// it by the state at the chunk's start, carrying decay^(rows of the chunk)
+// across each chunk. chunk_rows[k] = rows of chunk k.
+__global__ __launch_bounds__(256) void lightning_combine_kernel(
+    float* __restrict__ part, const float* __restrict__ decay,
+    float* __restrict__ state, const int* __restrict__ chunk_off,
+    const int* __restrict__ chunk_rows, const int* __restrict__ cu,
+    const int* __restrict__ seq_lens, const int* __restrict__ slots, int H,
+    int DV) {
+  const int s = blockIdx.y;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (int64_t)H * DV) return;
+  const int rows = cu[s + 1] - cu[s];
+  if (rows == 0) return;
+  const int start = seq_lens[s] - rows;
+  const int slot = slots[s];
+  const float lam = decay[e / DV];
+  float carry = (start > 0 && slot >= 0) ? state[(int64_t)slot * H * DV + e] : 0.f;
+  for (int k = chunk_off[s]; k < chunk_off[s + 1]; ++k) {
+    float* p = part + (int64_t)k * H * DV + e;
+    const float local = *p;
+    *p = carry;
+    carry = powf(lam, (float)chunk_rows[k]) * carry + local;
+  }
+  if (slot >= 0) state[(int64_t)slot * H * DV + e] = carry;
+}
+
 }  // namespace arks
 
 using namespace arks;
+
+extern "C" void arks_seq_lightning_combine(void* part, const void* decay,
+                                           void* state, const void* chunk_off,
+                                           const void* chunk_rows,
+                                           const void* cu, const void* seq_lens,
+                                           const void* slots, int S, int H,
+                                           int DV, hipStream_t stream) {
+  if (S == 0) return;
+  const int64_t n = (int64_t)H * DV;
+  hipLaunchKernelGGL(lightning_combine_kernel,
+                     dim3((unsigned)((n + 255) / 256), S), dim3(256), 0, stream,
+                     (float*)part, (const float*)decay, (float*)state,
+                     (const int*)chunk_off, (const int*)chunk_rows,
+                     (const int*)cu, (const int*)seq_lens, (const int*)slots, H,
+                     DV);
+}
 
 template <typename AT>
 static int launch_lightning(float* out, const void* q, const void* k,

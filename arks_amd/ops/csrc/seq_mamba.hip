@@ -73,9 +73,12 @@ __global__ __launch_bounds__(256) void conv_state_update_kernel(
     if (i < nh) hist[(int64_t)i * C] = nv[i];
 }
 
-// General selective scan: 16 lanes per channel (4 channels per wave), lane
-// ln owns states n = ln + 16 i. Rows are walked in order; dt's projection
-// and the output sum are reduced over the 16 lanes.
+// Selective scan: 16 lanes per channel (4 channels per wave), lane ln owns
+// states n = ln + 16 i. Rows are walked in order; the output sum is reduced
+// over the 16 lanes. dt's pre-activation either comes from a GEMM (dt_pre,
+// fp32 [T, C]) or is projected here from dt_raw. dsum (optional, [S, C])
+// receives each sequence's sum of dt — what the chunk-parallel prefill
+// needs to carry a state across a chunk: prod_t exp(dt_t A) = exp(A dsum).
 template <typename AT, int NPT>
 __global__ __launch_bounds__(64) void selective_scan_kernel(
     AT* __restrict__ out, const AT* __restrict__ u, const AT* __restrict__ dbc,
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
     const float* __restrict__ A, const float* __restrict__ Dp,
     float* __restrict__ state, const int* __restrict__ cu,
     const int* __restrict__ seq_lens, const int* __restrict__ slots, int C,
-    int N, int R) {
+    int N, int R, const float* __restrict__ dt_pre, float* __restrict__ dsum) {
   const int s = blockIdx.y;
   const int c = blockIdx.x * 4 + threadIdx.x / 16;
   const int ln = threadIdx.x % 16;
@@ -105,12 +108,20 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
   }
   const float dtb = dt_b[cc], dd = Dp[cc];
   const float* wr = dt_w + (int64_t)cc * R;
+  float dts = 0.f;
   for (int r = 0; r < rows; ++r) {
     const int t = a + r;
     const AT* drow = dbc + (int64_t)t * ldd;
-    float dtp = 0.f;
-    for (int j = ln; j < R; j += 16) dtp += wr[j] * Act<AT>::ld(drow + j);
-    const float dt = softplus_f(group16_reduce_sum(dtp) + dtb);
+    float dtp;
+    if (dt_pre) {
+      dtp = dt_pre[(int64_t)t * C + cc];
+    } else {
+      dtp = 0.f;
+      for (int j = ln; j < R; j += 16) dtp += wr[j] * Act<AT>::ld(drow + j);
+      dtp = group16_reduce_sum(dtp);
+    }
+    const float dt = softplus_f(dtp + dtb);
+    dts += dt;
     const float xv = Act<AT>::ld(u + (int64_t)t * C + cc);
     const float dx = dt * xv;
     float y = 0.f;
@@ -137,6 +148,38 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
       if (n < N) sp[n] = S[i];
     }
   }
+  if (dsum && ln == 0 && live) dsum[(int64_t)s * C + c] = dts;
+}
+
+// Chunk-parallel prefill, middle step. Each sequence's rows were cut into
+// chunks and scanned from zero state: part[k] holds chunk k's end state,
+// dsum[k] its sum of dt. Walk a sequence's chunks in order, one thread per
+// (channel, state): part[k] is replaced by the state at the START of chunk
+// k (what the final pass scans from) and the sequence's slot receives the
+// state after its last row.
+__global__ __launch_bounds__(256) void scan_combine_kernel(
+    float* __restrict__ part, const float* __restrict__ dsum,
+    const float* __restrict__ A, float* __restrict__ state,
+    const int* __restrict__ chunk_off, const int* __restrict__ cu,
+    const int* __restrict__ seq_lens, const int* __restrict__ slots, int C,
+    int N) {
+  const int s = blockIdx.y;
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (int64_t)C * N) return;
+  const int c = (int)(e / N);
+  const int rows = cu[s + 1] - cu[s];
+  if (rows == 0) return;
+  const int start = seq_lens[s] - rows;
+  const int slot = slots[s];
+  const float a = A[e];
+  float carry = (start > 0 && slot >= 0) ? state[(int64_t)slot * C * N + e] : 0.f;
+  for (int k = chunk_off[s]; k < chunk_off[s + 1]; ++k) {
+    float* p = part + (int64_t)k * C * N + e;
+    const float local = *p;
+    *p = carry;
+    carry = expf(a * dsum[(int64_t)k * C + c]) * carry + local;
+  }
+  if (slot >= 0) state[(int64_t)slot * C * N + e] = carry;
 }
 
 }  // namespace arks
@@ -172,13 +215,13 @@ static int launch_scan(void* out, const void* u, const void* dbc, int64_t ldd,
                        const float* dt_b, const float* A, const float* Dp,
                        float* state, const int* cu, const int* seq_lens,
                        const int* slots, int S, int C, int N, int R,
-                       hipStream_t stream) {
+                       const float* dt_pre, float* dsum, hipStream_t stream) {
   dim3 grid((C + 3) / 4, S), block(64);
 #define SS(NP)                                                                \
   hipLaunchKernelGGL((selective_scan_kernel<AT, NP>), grid, block, 0, stream, \
                      (AT*)out, (const AT*)u, (const AT*)dbc, ldd,             \
                      (const AT*)z, ldz, dt_w, dt_b, A, Dp, state, cu,         \
-                     seq_lens, slots, C, N, R)
+                     seq_lens, slots, C, N, R, dt_pre, dsum)
   if (N <= 16) SS(1);
   else if (N <= 32) SS(2);
   else if (N <= 64) SS(4);
@@ -193,13 +236,29 @@ extern "C" int arks_seq_selective_scan(
     void* out, const void* u, const void* dbc, int64_t ldd, const void* z,
     int64_t ldz, const void* dt_w, const void* dt_b, const void* A,
     const void* Dp, void* state, const void* cu, const void* seq_lens,
-    const void* slots, int S, int C, int N, int R, int act_f32,
-    hipStream_t stream) {
+    const void* slots, int S, int C, int N, int R, const void* dt_pre,
+    void* dsum, int act_f32, hipStream_t stream) {
   if (S == 0) return 0;
   int rc = 0;
   SEQ_DISPATCH_ACT(act_f32, rc = launch_scan<AT>(
       out, u, dbc, ldd, z, ldz, (const float*)dt_w, (const float*)dt_b,
       (const float*)A, (const float*)Dp, (float*)state, (const int*)cu,
-      (const int*)seq_lens, (const int*)slots, S, C, N, R, stream));
+      (const int*)seq_lens, (const int*)slots, S, C, N, R,
+      (const float*)dt_pre, (float*)dsum, stream));
   return rc;
+}
+
+extern "C" void arks_seq_scan_combine(void* part, const void* dsum,
+                                      const void* A, void* state,
+                                      const void* chunk_off, const void* cu,
+                                      const void* seq_lens, const void* slots,
+                                      int S, int C, int N,
+                                      hipStream_t stream) {
+  if (S == 0) return;
+  const int64_t n = (int64_t)C * N;
+  hipLaunchKernelGGL(scan_combine_kernel, dim3((unsigned)((n + 255) / 256), S),
+                     dim3(256), 0, stream, (float*)part, (const float*)dsum,
+                     (const float*)A, (float*)state, (const int*)chunk_off,
+                     (const int*)cu, (const int*)seq_lens, (const int*)slots,
+                     C, N);
 }

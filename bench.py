@@ -77,12 +77,17 @@ def run_cold_start(args):
         save_random_checkpoint(mcfg, ckpt, seed=args.seed)
     nbytes = sum(os.path.getsize(f)
                  for f in glob.glob(os.path.join(ckpt, "*.safetensors")))
-    # drop the page cache so the read really comes from disk
+    # evict this checkpoint's pages from the page cache (per file, no
+    # machine-wide setting) so the read really comes from disk
+    cache_dropped = True
     try:
         subprocess.run(["sync"], check=False)
-        with open("/proc/sys/vm/drop_caches", "w") as f:
-            f.write("3\n")
-        cache_dropped = True
+        for f in glob.glob(os.path.join(ckpt, "*.safetensors")):
+            fd = os.open(f, os.O_RDONLY)
+            try:
+                os.posix_fadvise(fd, 0, 0, os.POSIX_FADV_DONTNEED)
+            finally:
+                os.close(fd)
     except OSError:
         cache_dropped = False
     cfg = EngineConfig(

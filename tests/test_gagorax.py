@@ -268,3 +268,29 @@ def test_attention_head_sizes_of_the_mfma_kernels(tmp_path, device, dtype, dim, 
     got = replay(eng, tmp_path, steps)
     assert rel_err(got["a"], orc.run(ta)) < TOL[dtype]
     assert rel_err(got["b"], orc.run(tb)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_long_portions_cross_the_recurrent_chunks(tmp_path, device, dtype):
+    """Portions longer than one chunk of the chunk-parallel recurrent
+    prefill (64 rows): one row more, exact multiples, one row less, beside
+    a second request and single tokens."""
+    w = write_checkpoint(tmp_path / "m", MIXED, seed=4)
+    orc = Oracle(MIXED, w)
+    ta, tb = toks(330, seed=31), toks(200, seed=32)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=576)
+    cuts_a = [65, 128, 1, 63, 73]
+    steps, at = [], 0
+    for k, n in enumerate(cuts_a):
+        st = [("a", ta[at:at + n], at + n == 330)]
+        if k == 1:
+            st.append(("b", tb[:129], False))
+        if k == 2:
+            st.append(("b", tb[129:130], False))
+        if k == 3:
+            st.append(("b", tb[130:], True))
+        steps.append(st)
+        at += n
+    got = replay(eng, tmp_path, steps)
+    assert rel_err(got["a"], orc.run(ta)) < TOL[dtype]
+    assert rel_err(got["b"], orc.run(tb)) < TOL[dtype]

@@ -229,3 +229,53 @@ def test_selective_scan_remembers_through_a_slow_channel(dev, dtype):
         assert abs(float(last[0]) - want0) < 0.02 * want0
         assert abs(float(last[1])) < 1e-6
         assert float(state[1].min()) == 5.0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("lens", [[65], [64, 1, 200], [129, 128, 63]])
+def test_chunk_parallel_scans_equal_row_by_row(dtype, lens):
+    """The chunk-parallel prefill of both recurrent mixers against the same
+    kernels walking every row in order, with old state in the slots."""
+    dev = "cuda"
+    torch.manual_seed(sum(lens))
+    T, S = sum(lens), len(lens)
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    starts = [0, 7, 300][:S]
+    seq_lens = [s + n for s, n in zip(starts, lens)]
+    slots = [2, 0, 3][:S]
+    meta = (i32(cu, dev), i32(seq_lens, dev), i32(slots, dev))
+    chunks = ops.scan_chunks(lens, torch.device(dev))
+    # lightning
+    H, D, V = 3, 16, 24
+    q, k, v = (torch.randn(T, H, n, device=dev).to(dtype) for n in (D, D, V))
+    decay = torch.tensor([1.0, 0.97, 0.6], device=dev)
+    st0 = torch.randn(4, H, D, V, device=dev)
+    sa, sb = st0.clone(), st0.clone()
+    a = ops.lightning_scan(q, k, v, decay, sa, *meta, max_q_len=max(lens))
+    b = ops.lightning_scan(q, k, v, decay, sb, *meta, max_q_len=max(lens), chunks=chunks)
+    assert torch.allclose(a, b, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(sa, sb, rtol=1e-4, atol=1e-4)
+    # selective scan, with dt from a GEMM and projected in the kernel
+    C, N, R = 40, 12, 5
+    u = torch.randn(T, C, device=dev).to(dtype)
+    dbc = torch.randn(T, R + 2 * N, device=dev).to(dtype)
+    z = torch.randn(T, C, device=dev).to(dtype)
+    dt_w = torch.randn(C, R, device=dev) * 0.3
+    dt_b = torch.randn(C, device=dev) - 1.0
+    A = -torch.rand(C, N, device=dev) * 2
+    Dp = torch.randn(C, device=dev)
+    st0 = torch.randn(4, C, N, device=dev)
+    dt_pre = dbc[:, :R].float() @ dt_w.t()
+    outs = []
+    for kw in ({}, {"chunks": chunks}, {"dt_pre": dt_pre, "chunks": chunks}):
+        st = st0.clone()
+        y = ops.selective_scan(u, dbc, z, dt_w, dt_b, A, Dp, st, *meta,
+                               max_q_len=max(lens), **kw)
+        outs.append((y.float(), st))
+    tol = 2e-2 if dtype == torch.bfloat16 else 2e-4
+    for y, st in outs[1:]:
+        assert torch.allclose(y, outs[0][0], rtol=tol, atol=tol)
+        assert torch.allclose(st, outs[0][1], rtol=1e-4, atol=1e-4)
