@@ -151,6 +151,75 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
   if (dsum && ln == 0 && live) dsum[(int64_t)s * C + c] = dts;
 }
 
+// Selective scan for small state sizes with dt from a GEMM: one LANE per
+// channel, its N states in registers. A wave reads 64 consecutive channels
+// of u / dt_pre / z per row (coalesced), B and C of the row are the same
+// for every lane (uniform loads), and the sum over states stays inside the
+// lane — no shuffles, 16x fewer waves than the lane-split kernel above for
+// N = 16. Same arguments and state handling as selective_scan_kernel.
+template <typename AT, int NMAX>
+__global__ __launch_bounds__(64) void selective_scan_lane_kernel(
+    AT* __restrict__ out, const AT* __restrict__ u, const AT* __restrict__ dbc,
+    int64_t ldd, const AT* __restrict__ z, int64_t ldz,
+    const float* __restrict__ dt_b, const float* __restrict__ A,
+    const float* __restrict__ Dp, float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ seq_lens,
+    const int* __restrict__ slots, int C, int N, int R,
+    const float* __restrict__ dt_pre, float* __restrict__ dsum) {
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * 64 + threadIdx.x;
+  const int a = cu[s], rows = cu[s + 1] - a;
+  if (rows == 0) return;
+  const bool live = c < C;
+  const int cc = live ? c : C - 1;
+  const int start = seq_lens[s] - rows;
+  const int slot = slots[s];
+  const bool has_state = start > 0 && slot >= 0;
+  float* sp = state + ((int64_t)(slot < 0 ? 0 : slot) * C + cc) * N;
+  float S[NMAX], Av[NMAX];
+#pragma unroll
+  for (int n = 0; n < NMAX; ++n) {
+    S[n] = (has_state && n < N) ? sp[n] : 0.f;
+    Av[n] = n < N ? A[(int64_t)cc * N + n] : 0.f;
+  }
+  const float dtb = dt_b[cc], dd = Dp[cc];
+  float dts = 0.f;
+  // one row ahead: the next row's operands are in flight while this row's
+  // recurrence runs
+  float dtp_n = dt_pre[(int64_t)a * C + cc];
+  float xv_n = Act<AT>::ld(u + (int64_t)a * C + cc);
+  float zv_n = Act<AT>::ld(z + (int64_t)a * ldz + cc);
+  for (int r = 0; r < rows; ++r) {
+    const int t = a + r;
+    const float dtp = dtp_n, xv = xv_n, zv = zv_n;
+    if (r + 1 < rows) {
+      dtp_n = dt_pre[(int64_t)(t + 1) * C + cc];
+      xv_n = Act<AT>::ld(u + (int64_t)(t + 1) * C + cc);
+      zv_n = Act<AT>::ld(z + (int64_t)(t + 1) * ldz + cc);
+    }
+    const AT* brow = dbc + (int64_t)t * ldd + R;  // [B | C], uniform
+    const float dt = softplus_f(dtp + dtb);
+    dts += dt;
+    const float dx = dt * xv;
+    float y = 0.f;
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n) {
+      if (n < N) {
+        S[n] = expf(dt * Av[n]) * S[n] + dx * Act<AT>::ld(brow + n);
+        y += S[n] * Act<AT>::ld(brow + N + n);
+      }
+    }
+    if (live)
+      Act<AT>::st(out + (int64_t)t * C + c, (y + dd * xv) * silu_f(zv));
+  }
+  if (slot >= 0 && live) {
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n)
+      if (n < N) sp[n] = S[n];
+  }
+  if (dsum && live) dsum[(int64_t)s * C + c] = dts;
+}
+
 // Chunk-parallel prefill, middle step. Each sequence's rows were cut into
 // chunks and scanned from zero state: part[k] holds chunk k's end state,
 // dsum[k] its sum of dt. Walk a sequence's chunks in order, one thread per
@@ -216,6 +285,20 @@ static int launch_scan(void* out, const void* u, const void* dbc, int64_t ldd,
                        float* state, const int* cu, const int* seq_lens,
                        const int* slots, int S, int C, int N, int R,
                        const float* dt_pre, float* dsum, hipStream_t stream) {
+  if (dt_pre && N <= 64) {
+    dim3 lgrid((C + 63) / 64, S);
+#define SL(NM)                                                                 \
+  hipLaunchKernelGGL((selective_scan_lane_kernel<AT, NM>), lgrid, dim3(64), 0, \
+                     stream, (AT*)out, (const AT*)u, (const AT*)dbc, ldd,      \
+                     (const AT*)z, ldz, dt_b, A, Dp, state, cu, seq_lens,      \
+                     slots, C, N, R, dt_pre, dsum)
+    if (N <= 8) SL(8);
+    else if (N <= 16) SL(16);
+    else if (N <= 32) SL(32);
+    else SL(64);
+#undef SL
+    return 0;
+  }
   dim3 grid((C + 3) / 4, S), block(64);
 #define SS(NP)                                                                \
   hipLaunchKernelGGL((selective_scan_kernel<AT, NP>), grid, block, 0, stream, \
