@@ -211,6 +211,8 @@ class Mamba1Mixer(nn.Module):
         # in place from the fp32 dt_w: tiny ranks, CPU reference)
         self.register_buffer("dt_w_mm", torch.zeros(inner, dt_rank, dtype=dtype),
                              persistent=False)
+        self.register_buffer("conv_w_t", torch.zeros(conv, inner, dtype=f32),
+                             persistent=False)
 
     def weight_map(self) -> dict:
         return {"in": (self.w_in, 0), "x": (self.w_x, 0), "o": (self.o, 0),
@@ -221,6 +223,7 @@ class Mamba1Mixer(nn.Module):
     def finish_loading(self) -> None:
         self.A.copy_(-torch.exp(self.A_log.data.float()))
         self.dt_w_mm.copy_(self.dt_w.data)
+        self.conv_w_t.copy_(self.conv_w.data.t())
 
     def cache_layout(self, block_size: int, dtype) -> dict:
         out = {"ssm": ("slot", (self.C, self.N), torch.float32)}
@@ -234,7 +237,7 @@ class Mamba1Mixer(nn.Module):
         u = ops.causal_conv_silu(
             xz[:, :C], self.conv_w, self.conv_b, cache.get("conv"),
             batch.cu_seqlens, batch.seq_lens, batch.state_slots,
-            batch.token_seq)
+            batch.token_seq, self.conv_w_t)
         dbc = linear(u, self.w_x)
         dt_pre = None
         if xs.is_cuda and self.R >= 8:

@@ -769,11 +769,13 @@ def gated_rmsnorm(o, weight, gate, eps, out_dtype):
 
 
 def causal_conv_silu(x, weight, bias, state, cu_seqlens, seq_lens,
-                     state_slots, token_seq):
+                     state_slots, token_seq, weight_t=None):
+    """weight_t: [taps, C] copy of the taps for the vectorised bf16 kernel."""
     if x.is_cuda:
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-        _native_seq().causal_conv_silu(out, x, weight, bias, state, cu_seqlens,
-                                       seq_lens, state_slots, token_seq)
+        _native_seq().causal_conv_silu(out, x, weight, weight_t, bias, state,
+                                       cu_seqlens, seq_lens, state_slots,
+                                       token_seq)
         return out
     return ref.causal_conv_silu(x, weight, bias, state, cu_seqlens, seq_lens,
                                 state_slots)
@@ -793,8 +795,12 @@ def selective_scan(u, dbc, z, dt_w, dt_b, A, Dp, state, cu_seqlens, seq_lens,
                                device=u.device)
             dsum = torch.empty((c["n"], C), dtype=torch.float32,
                                device=u.device)
-            S.selective_scan(out, u, dbc, z, dt_w, dt_b, A, Dp, part, c["cu"],
-                             c["lens0"], c["slots"], dt_pre, dsum)
+            # pass 1 needs end states and dt sums only: the lane kernel
+            # skips the outputs when it is given none
+            light = dt_pre is not None and N <= 64
+            S.selective_scan(None if light else out, u, dbc, z, dt_w, dt_b, A,
+                             Dp, part, c["cu"], c["lens0"], c["slots"], dt_pre,
+                             dsum)
             S.scan_combine(part, dsum, A, state, c["off"], cu_seqlens,
                            seq_lens, state_slots)
             S.selective_scan(out, u, dbc, z, dt_w, dt_b, A, Dp, part, c["cu"],

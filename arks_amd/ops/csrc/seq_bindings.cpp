@@ -44,7 +44,8 @@ int arks_seq_lightning_scan(void* out, const void* q, const void* k,
                             const void* slots, int S, int H, int D, int V,
                             int act_f32, hipStream_t stream);
 int arks_seq_causal_conv_silu(void* out, const void* x, int64_t ldx,
-                              const void* w, const void* bias, void* state,
+                              const void* w, const void* w_t, const void* bias,
+                              void* state,
                               const void* cu, const void* seq_lens,
                               const void* slots, const void* token_seq, int T,
                               int S, int C, int taps, int act_f32,
@@ -354,9 +355,9 @@ void lightning_scan(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
   TORCH_CHECK(rc == 0, "lightning head size beyond the kernel's limit (", D, ")");
 }
 
-void causal_conv_silu(Tensor out, Tensor x, Tensor w, Tensor bias,
-                      OptTensor state, Tensor cu, Tensor seq_lens, Tensor slots,
-                      Tensor token_seq) {
+void causal_conv_silu(Tensor out, Tensor x, Tensor w, OptTensor w_t,
+                      Tensor bias, OptTensor state, Tensor cu, Tensor seq_lens,
+                      Tensor slots, Tensor token_seq) {
   const int f32 = act_flag(x, "x");
   const int T = x.size(0), C = x.size(1);
   TORCH_CHECK(out.scalar_type() == x.scalar_type() && out.is_contiguous() &&
@@ -365,6 +366,12 @@ void causal_conv_silu(Tensor out, Tensor x, Tensor w, Tensor bias,
   check_f32(bias, "conv bias");
   TORCH_CHECK(w.dim() == 2 && w.size(0) == C && bias.numel() == C);
   const int taps = w.size(1);
+  const void* wt_p = nullptr;
+  if (w_t.has_value()) {  // [taps, C] copy for the vectorised kernel
+    check_f32(*w_t, "transposed conv weight");
+    TORCH_CHECK(w_t->dim() == 2 && w_t->size(0) == taps && w_t->size(1) == C);
+    wt_p = w_t->data_ptr();
+  }
   void* st_p = nullptr;
   if (taps > 1) {
     TORCH_CHECK(state.has_value());
@@ -375,21 +382,30 @@ void causal_conv_silu(Tensor out, Tensor x, Tensor w, Tensor bias,
   }
   const SeqMeta m = check_meta(cu, seq_lens, &slots, &token_seq, T);
   const int rc = arks_seq_causal_conv_silu(
-      out.data_ptr(), x.data_ptr(), row_stride(x, "x"), w.data_ptr(),
+      out.data_ptr(), x.data_ptr(), row_stride(x, "x"), w.data_ptr(), wt_p,
       bias.data_ptr(), st_p, cu.data_ptr(), seq_lens.data_ptr(),
       slots.data_ptr(), token_seq.data_ptr(), T, m.S, C, taps, f32,
       current_stream());
   TORCH_CHECK(rc == 0, "conv taps beyond the kernel's limit (", taps, ")");
 }
 
-void selective_scan(Tensor out, Tensor u, Tensor dbc, Tensor z, Tensor dt_w,
+void selective_scan(OptTensor out_, Tensor u, Tensor dbc, Tensor z, Tensor dt_w,
                     Tensor dt_b, Tensor A, Tensor Dp, Tensor state, Tensor cu,
                     Tensor seq_lens, Tensor slots, OptTensor dt_pre,
                     OptTensor dsum) {
   const int f32 = act_flag(u, "u");
   const int T = u.size(0), C = u.size(1);
-  TORCH_CHECK(u.is_contiguous() && out.is_contiguous() &&
-              out.scalar_type() == u.scalar_type() && out.sizes() == u.sizes());
+  TORCH_CHECK(u.is_contiguous());
+  void* out_p = nullptr;  // none: state-only pass (needs dt_pre, N <= 64)
+  if (out_.has_value()) {
+    const Tensor& out = *out_;
+    TORCH_CHECK(out.is_contiguous() && out.scalar_type() == u.scalar_type() &&
+                out.sizes() == u.sizes());
+    out_p = out.data_ptr();
+  } else {
+    TORCH_CHECK(dt_pre.has_value() && A.size(1) <= 64,
+                "a state-only scan needs dt_pre and a state size <= 64");
+  }
   TORCH_CHECK(dbc.scalar_type() == u.scalar_type() &&
               z.scalar_type() == u.scalar_type());
   check_f32(dt_w, "dt weight");
@@ -420,7 +436,7 @@ void selective_scan(Tensor out, Tensor u, Tensor dbc, Tensor z, Tensor dt_w,
     dsum_p = dsum->data_ptr();
   }
   const int rc = arks_seq_selective_scan(
-      out.data_ptr(), u.data_ptr(), dbc.data_ptr(), row_stride(dbc, "dbc"),
+      out_p, u.data_ptr(), dbc.data_ptr(), row_stride(dbc, "dbc"),
       z.data_ptr(), row_stride(z, "z"), dt_w.data_ptr(), dt_b.data_ptr(),
       A.data_ptr(), Dp.data_ptr(), state.data_ptr(), cu.data_ptr(),
       seq_lens.data_ptr(), slots.data_ptr(), m.S, C, N, R, dtp_p, dsum_p, f32,

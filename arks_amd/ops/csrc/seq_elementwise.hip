@@ -62,6 +62,108 @@ __global__ __launch_bounds__(256) void gated_norm_residual_kernel(
   }
 }
 
+// bf16 rows, 8 elements per thread and iteration, the gated values kept in
+// registers between the two passes (W <= 8 * 256 * GNR_VPT).
+constexpr int GNR_VPT = 4;
+
+__global__ __launch_bounds__(256) void gated_norm_residual_vec8_kernel(
+    float* __restrict__ x, bf16* __restrict__ xa, const bf16* __restrict__ y,
+    const bf16* __restrict__ g, int64_t ldg, const float* __restrict__ gb,
+    const float* __restrict__ w, float eps, int W) {
+  __shared__ float scratch[4];
+  const int t = blockIdx.x;
+  const bf16* yr = y + (int64_t)t * W;
+  const bf16* gr = g ? g + (int64_t)t * ldg : nullptr;
+  float z[GNR_VPT][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < GNR_VPT; ++k) {
+    const int i = (k * 256 + threadIdx.x) * 8;
+    if (i < W) {
+      const ushort8 yv = *reinterpret_cast<const ushort8*>(yr + i);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) z[k][e] = bf16_bits_to_float(yv[e]);
+      if (gr) {
+        const ushort8 gv = *reinterpret_cast<const ushort8*>(gr + i);
+        const float4v b0 = *reinterpret_cast<const float4v*>(gb + i);
+        const float4v b1 = *reinterpret_cast<const float4v*>(gb + i + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          z[k][e] *= sigmoid_f(bf16_bits_to_float(gv[e]) + (e < 4 ? b0[e] : b1[e - 4]));
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += z[k][e] * z[k][e];
+    }
+  }
+  ss = block_reduce_sum<256>(ss, scratch);
+  const float rstd = 1.f / sqrtf(ss / (float)W + eps);
+  float* xr = x + (int64_t)t * W;
+#pragma unroll
+  for (int k = 0; k < GNR_VPT; ++k) {
+    const int i = (k * 256 + threadIdx.x) * 8;
+    if (i < W) {
+      float4v x0 = *reinterpret_cast<const float4v*>(xr + i);
+      float4v x1 = *reinterpret_cast<const float4v*>(xr + i + 4);
+      const float4v w0 = *reinterpret_cast<const float4v*>(w + i);
+      const float4v w1 = *reinterpret_cast<const float4v*>(w + i + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x0[e] += z[k][e] * rstd * w0[e];
+        x1[e] += z[k][4 + e] * rstd * w1[e];
+      }
+      *reinterpret_cast<float4v*>(xr + i) = x0;
+      *reinterpret_cast<float4v*>(xr + i + 4) = x1;
+      if (xa) {
+        ushort8 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o[e] = float_to_bf16_bits(x0[e]);
+          o[4 + e] = float_to_bf16_bits(x1[e]);
+        }
+        *reinterpret_cast<ushort8*>(xa + (int64_t)t * W + i) = o;
+      }
+    }
+  }
+}
+
+// token shift, bf16 outputs, 8 elements per thread (W % 8 == 0)
+__global__ __launch_bounds__(256) void token_shift_vec8_kernel(
+    bf16* __restrict__ xs, bf16* __restrict__ xa, const float* __restrict__ x,
+    const float* __restrict__ w, float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ seq_lens,
+    const int* __restrict__ slots, const int* __restrict__ token_seq, int W) {
+  const int t = blockIdx.x;
+  const SeqRow r = seq_row(t, token_seq, cu, seq_lens, slots);
+  const bool first = (t == r.first_row);
+  const bool has_state = r.start > 0 && r.slot >= 0;
+  const float* xr = x + (int64_t)t * W;
+  const float* xp = first ? (state + (int64_t)(r.slot < 0 ? 0 : r.slot) * W)
+                          : x + (int64_t)(t - 1) * W;
+  const bool zero_prev = first && !has_state;
+  const float* xl = x + (int64_t)(r.first_row + r.rows - 1) * W;
+  for (int i = threadIdx.x * 8; i < W; i += 256 * 8) {
+    ushort8 os, oa;
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+      const int j = i + 4 * hlf;
+      const float4v xv = *reinterpret_cast<const float4v*>(xr + j);
+      float4v pv = {0.f, 0.f, 0.f, 0.f};
+      if (!zero_prev) pv = *reinterpret_cast<const float4v*>(xp + j);
+      const float4v wv = *reinterpret_cast<const float4v*>(w + j);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        os[4 * hlf + e] = float_to_bf16_bits(xv[e] + (pv[e] - xv[e]) * wv[e]);
+        oa[4 * hlf + e] = float_to_bf16_bits(xv[e]);
+      }
+      if (first && r.slot >= 0)
+        *reinterpret_cast<float4v*>(state + (int64_t)r.slot * W + j) =
+            *reinterpret_cast<const float4v*>(xl + j);
+    }
+    *reinterpret_cast<ushort8*>(xs + (int64_t)t * W + i) = os;
+    *reinterpret_cast<ushort8*>(xa + (int64_t)t * W + i) = oa;
+  }
+}
+
 // out = rmsnorm(x) * w [* sigmoid(gate)], x fp32.
 template <typename AT>
 __global__ __launch_bounds__(256) void rms_norm_f32_kernel(
@@ -210,6 +312,13 @@ extern "C" void arks_seq_token_shift(void* xs, void* xa, const void* x,
                                      const void* token_seq, int T, int W,
                                      int act_f32, hipStream_t stream) {
   if (T == 0) return;
+  if (!act_f32 && xa && W % 8 == 0) {
+    hipLaunchKernelGGL(token_shift_vec8_kernel, dim3(T), dim3(256), 0, stream,
+                       (bf16*)xs, (bf16*)xa, (const float*)x, (const float*)w,
+                       (float*)state, (const int*)cu, (const int*)seq_lens,
+                       (const int*)slots, (const int*)token_seq, W);
+    return;
+  }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (token_shift_kernel<AT>), dim3(T), dim3(256), 0, stream, (AT*)xs,
       (AT*)xa, (const float*)x, (const float*)w, (float*)state, (const int*)cu,
@@ -222,6 +331,14 @@ extern "C" void arks_seq_gated_norm_residual(void* x, void* xa, const void* y,
                                              float eps, int T, int W,
                                              int act_f32, hipStream_t stream) {
   if (T == 0) return;
+  if (!act_f32 && W % 8 == 0 && W <= 8 * 256 * GNR_VPT && ldg % 8 == 0 &&
+      ((uintptr_t)g % 16) == 0) {
+    hipLaunchKernelGGL(gated_norm_residual_vec8_kernel, dim3(T), dim3(256), 0,
+                       stream, (float*)x, (bf16*)xa, (const bf16*)y,
+                       (const bf16*)g, ldg, (const float*)gb, (const float*)w,
+                       eps, W);
+    return;
+  }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (gated_norm_residual_kernel<AT>), dim3(T), dim3(256), 0, stream,
       (float*)x, (AT*)xa, (const AT*)y, (const AT*)g, ldg, (const float*)gb,

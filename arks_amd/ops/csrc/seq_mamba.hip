@@ -41,6 +41,60 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
   }
 }
 
+// bf16 rows, 8 channels per thread: 16-byte loads of each tap's row, conv
+// taps from a transposed copy of the weights (w_t [taps, C]) so that they
+// load as two float4 per tap.
+__global__ __launch_bounds__(256) void causal_conv_silu_vec8_kernel(
+    bf16* __restrict__ out, const bf16* __restrict__ x, int64_t ldx,
+    const float* __restrict__ w_t, const float* __restrict__ bias,
+    const float* __restrict__ state, const int* __restrict__ cu,
+    const int* __restrict__ seq_lens, const int* __restrict__ slots,
+    const int* __restrict__ token_seq, int C, int taps) {
+  const int t = blockIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c >= C) return;
+  const SeqRow r = seq_row(t, token_seq, cu, seq_lens, slots);
+  const int i = t - r.first_row;
+  const bool has_state = r.start > 0 && r.slot >= 0;
+  const float* hist = state + (int64_t)(r.slot < 0 ? 0 : r.slot) * (taps - 1) * C;
+  float acc[8];
+  {
+    const float4v b0 = *reinterpret_cast<const float4v*>(bias + c);
+    const float4v b1 = *reinterpret_cast<const float4v*>(bias + c + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { acc[e] = b0[e]; acc[4 + e] = b1[e]; }
+  }
+  for (int j = 0; j < taps; ++j) {
+    const int src = i - (taps - 1 - j);
+    float xv[8];
+    if (src >= 0) {
+      const ushort8 v = *reinterpret_cast<const ushort8*>(
+          x + (int64_t)(r.first_row + src) * ldx + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xv[e] = bf16_bits_to_float(v[e]);
+    } else if (has_state) {
+      const float* hp = hist + (int64_t)(src + taps - 1) * C + c;
+      const float4v h0 = *reinterpret_cast<const float4v*>(hp);
+      const float4v h1 = *reinterpret_cast<const float4v*>(hp + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { xv[e] = h0[e]; xv[4 + e] = h1[e]; }
+    } else {
+      continue;
+    }
+    const float4v w0 = *reinterpret_cast<const float4v*>(w_t + (int64_t)j * C + c);
+    const float4v w1 = *reinterpret_cast<const float4v*>(w_t + (int64_t)j * C + c + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc[e] += w0[e] * xv[e];
+      acc[4 + e] += w1[e] * xv[4 + e];
+    }
+  }
+  ushort8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = float_to_bf16_bits(silu_f(acc[e]));
+  *reinterpret_cast<ushort8*>(out + (int64_t)t * C + c) = o;
+}
+
 // New history of a sequence = the last taps-1 inputs after this step: rows
 // of this step where there are enough, older history shifted up otherwise.
 // One thread per (sequence, channel) reads all it needs before it writes.
@@ -152,13 +206,20 @@ __global__ __launch_bounds__(64) void selective_scan_kernel(
 }
 
 // Selective scan for small state sizes with dt from a GEMM: one LANE per
-// channel, its N states in registers. A wave reads 64 consecutive channels
-// of u / dt_pre / z per row (coalesced), B and C of the row are the same
-// for every lane (uniform loads), and the sum over states stays inside the
-// lane — no shuffles, 16x fewer waves than the lane-split kernel above for
-// N = 16. Same arguments and state handling as selective_scan_kernel.
-template <typename AT, int NMAX>
-__global__ __launch_bounds__(64) void selective_scan_lane_kernel(
+// channel, its N states in registers; a block of 256 threads covers 256
+// consecutive channels of one sequence (or chunk). Row operands u / dt_pre
+// / z are read coalesced across channels; B and C of the rows — the same
+// for every channel — are staged in LDS as floats, SCAN_ROWS rows at a
+// time, and read back as broadcasts. The sum over states stays inside the
+// lane: no shuffles, 16x fewer waves than the lane-split kernel above for
+// N = 16. bf16 serving folds log2(e) into A and uses the hardware exp2;
+// float rows keep the precise expf. WITH_Y = false is the first pass of the
+// chunk-parallel prefill: only the end state and the sum of dt are needed.
+// Same arguments and state handling as selective_scan_kernel.
+constexpr int SCAN_ROWS = 32;
+
+template <typename AT, int NMAX, bool WITH_Y>
+__global__ __launch_bounds__(256) void selective_scan_lane_kernel(
     AT* __restrict__ out, const AT* __restrict__ u, const AT* __restrict__ dbc,
     int64_t ldd, const AT* __restrict__ z, int64_t ldz,
     const float* __restrict__ dt_b, const float* __restrict__ A,
@@ -166,8 +227,10 @@ __global__ __launch_bounds__(64) void selective_scan_lane_kernel(
     const int* __restrict__ cu, const int* __restrict__ seq_lens,
     const int* __restrict__ slots, int C, int N, int R,
     const float* __restrict__ dt_pre, float* __restrict__ dsum) {
+  constexpr bool FAST = sizeof(AT) == 2;
+  __shared__ float bc_s[SCAN_ROWS][2 * NMAX];
   const int s = blockIdx.y;
-  const int c = blockIdx.x * 64 + threadIdx.x;
+  const int c = blockIdx.x * 256 + threadIdx.x;
   const int a = cu[s], rows = cu[s + 1] - a;
   if (rows == 0) return;
   const bool live = c < C;
@@ -181,36 +244,40 @@ __global__ __launch_bounds__(64) void selective_scan_lane_kernel(
   for (int n = 0; n < NMAX; ++n) {
     S[n] = (has_state && n < N) ? sp[n] : 0.f;
     Av[n] = n < N ? A[(int64_t)cc * N + n] : 0.f;
+    if (FAST) Av[n] *= 1.4426950408889634f;
   }
   const float dtb = dt_b[cc], dd = Dp[cc];
   float dts = 0.f;
-  // one row ahead: the next row's operands are in flight while this row's
-  // recurrence runs
-  float dtp_n = dt_pre[(int64_t)a * C + cc];
-  float xv_n = Act<AT>::ld(u + (int64_t)a * C + cc);
-  float zv_n = Act<AT>::ld(z + (int64_t)a * ldz + cc);
-  for (int r = 0; r < rows; ++r) {
-    const int t = a + r;
-    const float dtp = dtp_n, xv = xv_n, zv = zv_n;
-    if (r + 1 < rows) {
-      dtp_n = dt_pre[(int64_t)(t + 1) * C + cc];
-      xv_n = Act<AT>::ld(u + (int64_t)(t + 1) * C + cc);
-      zv_n = Act<AT>::ld(z + (int64_t)(t + 1) * ldz + cc);
+  for (int r0 = 0; r0 < rows; r0 += SCAN_ROWS) {
+    const int nr = min(SCAN_ROWS, rows - r0);
+    __syncthreads();  // the previous tile's readers are done
+    for (int i = threadIdx.x; i < nr * 2 * N; i += 256) {
+      const int rr = i / (2 * N), col = i - rr * 2 * N;
+      bc_s[rr][col < N ? col : NMAX + (col - N)] =
+          Act<AT>::ld(dbc + (int64_t)(a + r0 + rr) * ldd + R + col);
     }
-    const AT* brow = dbc + (int64_t)t * ldd + R;  // [B | C], uniform
-    const float dt = softplus_f(dtp + dtb);
-    dts += dt;
-    const float dx = dt * xv;
-    float y = 0.f;
+    __syncthreads();
+    for (int rr = 0; rr < nr; ++rr) {
+      const int t = a + r0 + rr;
+      const float dt = softplus_f(dt_pre[(int64_t)t * C + cc] + dtb);
+      const float xv = Act<AT>::ld(u + (int64_t)t * C + cc);
+      dts += dt;
+      const float dx = dt * xv;
+      float y = 0.f;
 #pragma unroll
-    for (int n = 0; n < NMAX; ++n) {
-      if (n < N) {
-        S[n] = expf(dt * Av[n]) * S[n] + dx * Act<AT>::ld(brow + n);
-        y += S[n] * Act<AT>::ld(brow + N + n);
+      for (int n = 0; n < NMAX; ++n) {
+        if (n < N) {
+          const float e = FAST ? __builtin_amdgcn_exp2f(dt * Av[n])
+                               : expf(dt * Av[n]);
+          S[n] = e * S[n] + dx * bc_s[rr][n];
+          if (WITH_Y) y += S[n] * bc_s[rr][NMAX + n];
+        }
+      }
+      if (WITH_Y && live) {
+        const float zv = Act<AT>::ld(z + (int64_t)t * ldz + cc);
+        Act<AT>::st(out + (int64_t)t * C + c, (y + dd * xv) * silu_f(zv));
       }
     }
-    if (live)
-      Act<AT>::st(out + (int64_t)t * C + c, (y + dd * xv) * silu_f(zv));
   }
   if (slot >= 0 && live) {
 #pragma unroll
@@ -256,14 +323,24 @@ __global__ __launch_bounds__(256) void scan_combine_kernel(
 using namespace arks;
 
 extern "C" int arks_seq_causal_conv_silu(
-    void* out, const void* x, int64_t ldx, const void* w, const void* bias,
-    void* state, const void* cu, const void* seq_lens, const void* slots,
-    const void* token_seq, int T, int S, int C, int taps, int act_f32,
-    hipStream_t stream) {
+    void* out, const void* x, int64_t ldx, const void* w, const void* w_t,
+    const void* bias, void* state, const void* cu, const void* seq_lens,
+    const void* slots, const void* token_seq, int T, int S, int C, int taps,
+    int act_f32, hipStream_t stream) {
   if (taps - 1 > CONV_MAX_HIST || taps < 1) return 1;
   if (T == 0) return 0;
   const int cb = (C + 255) / 256;
+  const bool vec8 = !act_f32 && w_t && C % 8 == 0 && ldx % 8 == 0 &&
+                    ((uintptr_t)x % 16) == 0;
   SEQ_DISPATCH_ACT(act_f32, {
+    if (vec8)
+      hipLaunchKernelGGL(causal_conv_silu_vec8_kernel,
+                         dim3(T, (C / 8 + 255) / 256), dim3(256), 0, stream,
+                         (bf16*)out, (const bf16*)x, ldx, (const float*)w_t,
+                         (const float*)bias, (const float*)state,
+                         (const int*)cu, (const int*)seq_lens,
+                         (const int*)slots, (const int*)token_seq, C, taps);
+    else
     hipLaunchKernelGGL((causal_conv_silu_kernel<AT>), dim3(T, cb), dim3(256), 0,
                        stream, (AT*)out, (const AT*)x, ldx, (const float*)w,
                        (const float*)bias, (const float*)state, (const int*)cu,
@@ -286,12 +363,21 @@ static int launch_scan(void* out, const void* u, const void* dbc, int64_t ldd,
                        const int* slots, int S, int C, int N, int R,
                        const float* dt_pre, float* dsum, hipStream_t stream) {
   if (dt_pre && N <= 64) {
-    dim3 lgrid((C + 63) / 64, S);
-#define SL(NM)                                                                 \
-  hipLaunchKernelGGL((selective_scan_lane_kernel<AT, NM>), lgrid, dim3(64), 0, \
-                     stream, (AT*)out, (const AT*)u, (const AT*)dbc, ldd,      \
-                     (const AT*)z, ldz, dt_b, A, Dp, state, cu, seq_lens,      \
-                     slots, C, N, R, dt_pre, dsum)
+    dim3 lgrid((C + 255) / 256, S);
+    const bool with_y = out != nullptr;
+#define SL(NM)                                                                \
+  do {                                                                        \
+    if (with_y)                                                               \
+      hipLaunchKernelGGL((selective_scan_lane_kernel<AT, NM, true>), lgrid,   \
+                         dim3(256), 0, stream, (AT*)out, (const AT*)u,        \
+                         (const AT*)dbc, ldd, (const AT*)z, ldz, dt_b, A, Dp, \
+                         state, cu, seq_lens, slots, C, N, R, dt_pre, dsum);  \
+    else                                                                      \
+      hipLaunchKernelGGL((selective_scan_lane_kernel<AT, NM, false>), lgrid,  \
+                         dim3(256), 0, stream, (AT*)out, (const AT*)u,        \
+                         (const AT*)dbc, ldd, (const AT*)z, ldz, dt_b, A, Dp, \
+                         state, cu, seq_lens, slots, C, N, R, dt_pre, dsum);  \
+  } while (0)
     if (N <= 8) SL(8);
     else if (N <= 16) SL(16);
     else if (N <= 32) SL(32);
