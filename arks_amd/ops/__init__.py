@@ -710,6 +710,7 @@ def attention_sink_paged(q, k_cache, v_cache, block_tables, seq_lens,
 
 
 SCAN_CHUNK = 64  # rows per chunk of the chunk-parallel recurrent prefill
+use_lightning_mfma = True  # tests switch it off to compare both paths
 
 
 def scan_chunks(q_lens: list[int], device, chunk: int = SCAN_CHUNK) -> dict:
@@ -746,12 +747,20 @@ def lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
             c = chunks
             part = torch.empty((c["n"], H, D, V), dtype=torch.float32,
                                device=q.device)
-            S.lightning_scan(out, q, k, v, decay, part, c["cu"], c["lens0"],
-                             c["slots"], SCAN_CHUNK)
+            # bf16 rows with head sizes the matrix-core kernels are built
+            # for run those; the general kernel does the same two passes
+            mfma = (q.dtype == torch.bfloat16 and use_lightning_mfma
+                    and S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 1))
+            if not mfma:
+                S.lightning_scan(out, q, k, v, decay, part, c["cu"],
+                                 c["lens0"], c["slots"], SCAN_CHUNK)
             S.lightning_combine(part, decay, state, c["off"], c["rows"],
                                 cu_seqlens, seq_lens, state_slots)
-            S.lightning_scan(out, q, k, v, decay, part, c["cu"], c["lens1"],
-                             c["slots"], SCAN_CHUNK)
+            if mfma:
+                S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 2)
+            else:
+                S.lightning_scan(out, q, k, v, decay, part, c["cu"],
+                                 c["lens1"], c["slots"], SCAN_CHUNK)
             return out
         S.lightning_scan(out, q, k, v, decay, state, cu_seqlens, seq_lens,
                          state_slots, max_q_len)

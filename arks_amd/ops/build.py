@@ -46,6 +46,7 @@ SEQ_SOURCES = [
     os.path.join(CSRC, "attn_extend2.hip"),
     os.path.join(CSRC, "attn_decode.hip"),
     os.path.join(CSRC, "seq_lightning.hip"),
+    os.path.join(CSRC, "seq_lightning_mfma.hip"),
     os.path.join(CSRC, "seq_mamba.hip"),
 ]
 

@@ -61,6 +61,11 @@ void arks_seq_scan_combine(void* part, const void* dsum, const void* A,
                            void* state, const void* chunk_off, const void* cu,
                            const void* seq_lens, const void* slots, int S,
                            int C, int N, hipStream_t stream);
+int arks_seq_lightning_mfma(void* out, void* part, const void* q, const void* k,
+                            const void* v, int64_t ldq, int64_t ldk,
+                            int64_t ldv, const void* decay, const void* cu,
+                            int chunks, int H, int D, int V, int pass,
+                            hipStream_t stream);
 void arks_seq_lightning_combine(void* part, const void* decay, void* state,
                                 const void* chunk_off, const void* chunk_rows,
                                 const void* cu, const void* seq_lens,
@@ -465,6 +470,34 @@ void scan_combine(Tensor part, Tensor dsum, Tensor A, Tensor state,
                         current_stream());
 }
 
+// One pass of the matrix-core lightning prefill over chunks of <= 64 rows
+// (cu = chunk row starts). pass 1 fills part with chunk end states, pass 2
+// reads chunk start states from part and writes out. False: no kernel for
+// these head sizes (the caller runs the general kernel).
+bool lightning_mfma(Tensor out, Tensor part, Tensor q, Tensor k, Tensor v,
+                    Tensor decay, Tensor cu, int64_t pass) {
+  TORCH_CHECK(q.is_cuda() && q.scalar_type() == torch::kBFloat16 &&
+              k.scalar_type() == torch::kBFloat16 &&
+              v.scalar_type() == torch::kBFloat16, "bf16 rows only");
+  const int T = q.size(0), H = q.size(1), D = q.size(2), V = v.size(2);
+  TORCH_CHECK(k.size(0) == T && k.size(1) == H && k.size(2) == D &&
+              v.size(0) == T && v.size(1) == H);
+  check_f32(out, "out");
+  check_f32(part, "part");
+  check_f32(decay, "decay");
+  check_i32(cu, "chunk starts");
+  const int chunks = cu.numel() - 1;
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H && out.size(2) == V);
+  TORCH_CHECK(part.dim() == 4 && part.size(0) == chunks && part.size(1) == H &&
+              part.size(2) == D && part.size(3) == V && decay.numel() == H);
+  TORCH_CHECK(pass == 1 || pass == 2);
+  return arks_seq_lightning_mfma(
+             out.data_ptr(), part.data_ptr(), q.data_ptr(), k.data_ptr(),
+             v.data_ptr(), head_row_stride(q, "q"), head_row_stride(k, "k"),
+             head_row_stride(v, "v"), decay.data_ptr(), cu.data_ptr(), chunks,
+             H, D, V, (int)pass, current_stream()) == 0;
+}
+
 void lightning_combine(Tensor part, Tensor decay, Tensor state,
                        Tensor chunk_off, Tensor chunk_rows, Tensor cu,
                        Tensor seq_lens, Tensor slots) {
@@ -505,4 +538,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("selective_scan", &selective_scan);
   m.def("scan_combine", &scan_combine);
   m.def("lightning_combine", &lightning_combine);
+  m.def("lightning_mfma", &lightning_mfma);
 }

@@ -1,0 +1,276 @@
+// Lightning attention prefill on the matrix cores (bf16 rows, gfx950):
+// the two scans of the chunk-parallel scheme (ops.scan_chunks) as 64-row
+// block products, one workgroup of 4 waves per (chunk, head).
+//
+//   pass 1  part[d][v] = sum_j decay^(n-1-j) k_j[d] v_j[v]      (n rows)
+//   pass 2  o_i = decay^(i+1) (q_i . S0) + sum_{j<=i} decay^(i-j) (q_i.k_j) v_j
+//
+// with S0 the chunk's start state left in `part` by lightning_combine.
+// q, k, v are silu'd in fp32 on the way into LDS and rounded to bf16 for
+// v_mfma_f32_16x16x32_bf16. Every fp32 quantity that meets a matrix
+// operand — the decayed keys of pass 1, the decayed score matrix and the
+// fp32 state of pass 2 — is split into a bf16 high and low part and
+// multiplied twice, so decays, scores and state keep ~16 mantissa bits
+// through the products; accumulation is fp32.
+//
+// Operand convention (as in attn_extend.hip): mfma(a, b) gives
+// D[m][n] = sum_k a[m][k] b[n][k]; a lane holds row (lane % 16) and k =
+// 8 (lane / 16) .. +7 of each 32-wide k step; the result lane holds column
+// n = lane % 16, rows m = 4 (lane / 16) + r. So every operand sits in LDS
+// with k contiguous: V, decayed K and the state are staged transposed.
+#include "seq_common.h"
+
+namespace arks {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 lm_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float lm_f32x4;
+
+constexpr int LM_ROWS = 64;  // rows per chunk (ops.SCAN_CHUNK)
+constexpr int LM_PAD = 8;    // bf16 elements of row padding in LDS
+
+__device__ __forceinline__ lm_f32x4 lm_mfma(const bf16* a, const bf16* b,
+                                            lm_f32x4 c) {
+  ushort8 ua = *reinterpret_cast<const ushort8*>(a);
+  ushort8 ub = *reinterpret_cast<const ushort8*>(b);
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+      *reinterpret_cast<lm_bf16x8*>(&ua), *reinterpret_cast<lm_bf16x8*>(&ub), c,
+      0, 0, 0);
+}
+
+__device__ __forceinline__ void split_bf16(float x, bf16& hi, bf16& lo) {
+  hi = float_to_bf16_bits(x);
+  lo = float_to_bf16_bits(x - bf16_bits_to_float(hi));
+}
+
+// decay^e for integer e >= 0 (0^0 = 1)
+__device__ __forceinline__ float decay_pow(float log2_decay, int e) {
+  return e == 0 ? 1.f : __builtin_amdgcn_exp2f(log2_decay * (float)e);
+}
+
+// ---- pass 1: end state of each chunk scanned from zero
+template <int D, int V>
+__global__ __launch_bounds__(256) void lightning_state_mfma_kernel(
+    float* __restrict__ part,  // [chunks, H, D, V]
+    const bf16* __restrict__ k, const bf16* __restrict__ v, int64_t ldk,
+    int64_t ldv, const float* __restrict__ decay, const int* __restrict__ cu,
+    int H) {
+  constexpr int LK = LM_ROWS + LM_PAD;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lm_smem[];
+  bf16* kt_hi = reinterpret_cast<bf16*>(lm_smem);  // [D][LK]
+  bf16* kt_lo = kt_hi + D * LK;                    // [D][LK]
+  bf16* vt = kt_lo + D * LK;                       // [V][LK]
+  const int ch = blockIdx.x, h = blockIdx.y;
+  const int row0 = cu[ch], n = cu[ch + 1] - row0;
+  const float l2 = log2f(decay[h]);
+  const int tid = threadIdx.x;
+  for (int i = tid; i < LM_ROWS * D; i += 256) {
+    const int j = i / D, d = i - j * D;
+    float x = 0.f;
+    if (j < n)
+      x = silu_f(bf16_bits_to_float(k[(int64_t)(row0 + j) * ldk + (int64_t)h * D + d])) *
+          decay_pow(l2, n - 1 - j);
+    split_bf16(x, kt_hi[d * LK + j], kt_lo[d * LK + j]);
+  }
+  for (int i = tid; i < LM_ROWS * V; i += 256) {
+    const int j = i / V, c = i - j * V;
+    float x = 0.f;
+    if (j < n)
+      x = silu_f(bf16_bits_to_float(v[(int64_t)(row0 + j) * ldv + (int64_t)h * V + c]));
+    vt[c * LK + j] = float_to_bf16_bits(x);
+  }
+  __syncthreads();
+  const int wave = tid / 64, lane = tid % 64, lq = lane % 16, la = lane / 16;
+  constexpr int DT = D / 16, VT = V / 16;
+  float* out = part + ((int64_t)ch * H + h) * D * V;
+  for (int dt = wave; dt < DT; dt += 4) {
+    lm_f32x4 acc[VT];
+#pragma unroll
+    for (int c = 0; c < VT; ++c) acc[c] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < LM_ROWS / 32; ++st) {
+      const int ko = st * 32 + 8 * la;
+      const bf16* ah = kt_hi + (dt * 16 + lq) * LK + ko;
+      const bf16* al = kt_lo + (dt * 16 + lq) * LK + ko;
+#pragma unroll
+      for (int c = 0; c < VT; ++c) {
+        const bf16* b = vt + (c * 16 + lq) * LK + ko;
+        acc[c] = lm_mfma(ah, b, acc[c]);
+        acc[c] = lm_mfma(al, b, acc[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < VT; ++c)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        out[(int64_t)(dt * 16 + 4 * la + r) * V + c * 16 + lq] = acc[c][r];
+  }
+}
+
+// ---- pass 2: outputs of each chunk from its start state
+template <int D, int V>
+__global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
+    float* __restrict__ out,         // [T, H, V] fp32
+    const float* __restrict__ part,  // [chunks, H, D, V] start states
+    const bf16* __restrict__ q, const bf16* __restrict__ k,
+    const bf16* __restrict__ v, int64_t ldq, int64_t ldk, int64_t ldv,
+    const float* __restrict__ decay, const int* __restrict__ cu, int H) {
+  constexpr int LD = D + LM_PAD;
+  constexpr int LK = LM_ROWS + LM_PAD;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lm_smem[];
+  bf16* qs = reinterpret_cast<bf16*>(lm_smem);  // [64][LD]
+  bf16* ks = qs + LM_ROWS * LD;                 // [64][LD]
+  bf16* vt = ks + LM_ROWS * LD;                 // [V][LK]
+  bf16* a_hi = vt + V * LK;                     // [64][LK]
+  bf16* a_lo = a_hi + LM_ROWS * LK;             // [64][LK]
+  bf16* st_hi = a_lo + LM_ROWS * LK;            // [V][LD]  state^T
+  bf16* st_lo = st_hi + V * LD;                 // [V][LD]
+  const int ch = blockIdx.x, h = blockIdx.y;
+  const int row0 = cu[ch], n = cu[ch + 1] - row0;
+  const float l2 = log2f(decay[h]);
+  const int tid = threadIdx.x;
+  for (int i = tid; i < LM_ROWS * D; i += 256) {
+    const int j = i / D, d = i - j * D;
+    float xq = 0.f, xk = 0.f;
+    if (j < n) {
+      xq = silu_f(bf16_bits_to_float(q[(int64_t)(row0 + j) * ldq + (int64_t)h * D + d]));
+      xk = silu_f(bf16_bits_to_float(k[(int64_t)(row0 + j) * ldk + (int64_t)h * D + d]));
+    }
+    qs[j * LD + d] = float_to_bf16_bits(xq);
+    ks[j * LD + d] = float_to_bf16_bits(xk);
+  }
+  for (int i = tid; i < LM_ROWS * V; i += 256) {
+    const int j = i / V, c = i - j * V;
+    float x = 0.f;
+    if (j < n)
+      x = silu_f(bf16_bits_to_float(v[(int64_t)(row0 + j) * ldv + (int64_t)h * V + c]));
+    vt[c * LK + j] = float_to_bf16_bits(x);
+  }
+  {
+    const float* sp = part + ((int64_t)ch * H + h) * D * V;
+    for (int i = tid; i < D * V; i += 256) {
+      const int d = i / V, c = i - d * V;
+      split_bf16(sp[i], st_hi[c * LD + d], st_lo[c * LD + d]);
+    }
+  }
+  __syncthreads();
+  const int wave = tid / 64, lane = tid % 64, lq = lane % 16, la = lane / 16;
+  // scores of this wave's 16 rows against all 64 keys, decayed and masked,
+  // into a_hi/a_lo[i][j] (each wave writes only its own rows)
+  const int irow = wave * 16 + lq;  // the row this lane's score column is
+#pragma unroll
+  for (int jt = 0; jt < LM_ROWS / 16; ++jt) {
+    lm_f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < D / 32; ++st) {
+      const int ko = st * 32 + 8 * la;
+      sc = lm_mfma(ks + (jt * 16 + lq) * LD + ko, qs + irow * LD + ko, sc);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int j = jt * 16 + 4 * la + r;
+      const float w = (j <= irow && irow < n) ? sc[r] * decay_pow(l2, irow - j) : 0.f;
+      split_bf16(w, a_hi[irow * LK + j], a_lo[irow * LK + j]);
+    }
+  }
+  __syncthreads();
+  constexpr int VT = V / 16;
+  lm_f32x4 acc[VT], acs[VT];
+#pragma unroll
+  for (int c = 0; c < VT; ++c) {
+    acc[c] = {0.f, 0.f, 0.f, 0.f};
+    acs[c] = {0.f, 0.f, 0.f, 0.f};
+  }
+  const int arow = wave * 16 + lq;  // A-operand row of this lane
+#pragma unroll
+  for (int st = 0; st < LM_ROWS / 32; ++st) {
+    const int ko = st * 32 + 8 * la;
+#pragma unroll
+    for (int c = 0; c < VT; ++c) {
+      const bf16* b = vt + (c * 16 + lq) * LK + ko;
+      acc[c] = lm_mfma(a_hi + arow * LK + ko, b, acc[c]);
+      acc[c] = lm_mfma(a_lo + arow * LK + ko, b, acc[c]);
+    }
+  }
+#pragma unroll
+  for (int st = 0; st < D / 32; ++st) {
+    const int ko = st * 32 + 8 * la;
+#pragma unroll
+    for (int c = 0; c < VT; ++c) {
+      acs[c] = lm_mfma(qs + arow * LD + ko, st_hi + (c * 16 + lq) * LD + ko, acs[c]);
+      acs[c] = lm_mfma(qs + arow * LD + ko, st_lo + (c * 16 + lq) * LD + ko, acs[c]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int i = wave * 16 + 4 * la + r;
+    if (i >= n) continue;
+    const float carry = decay_pow(l2, i + 1);
+    float* orow = out + ((int64_t)(row0 + i) * H + h) * V;
+#pragma unroll
+    for (int c = 0; c < VT; ++c) orow[c * 16 + lq] = acc[c][r] + carry * acs[c][r];
+  }
+}
+
+}  // namespace arks
+
+using namespace arks;
+
+template <int D, int V>
+static void launch_lm(float* out, float* part, const void* q, const void* k,
+                      const void* v, int64_t ldq, int64_t ldk, int64_t ldv,
+                      const float* decay, const int* cu, int chunks, int H,
+                      int pass, hipStream_t stream) {
+  constexpr int LD = D + LM_PAD, LK = LM_ROWS + LM_PAD;
+  dim3 grid(chunks, H), block(256);
+  if (pass == 1) {
+    constexpr int lds = (2 * D * LK + V * LK) * 2;
+    static bool set = false;
+    if (!set) {
+      (void)hipFuncSetAttribute(
+          reinterpret_cast<const void*>(lightning_state_mfma_kernel<D, V>),
+          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      set = true;
+    }
+    hipLaunchKernelGGL((lightning_state_mfma_kernel<D, V>), grid, block, lds,
+                       stream, part, (const bf16*)k, (const bf16*)v, ldk, ldv,
+                       decay, cu, H);
+  } else {
+    constexpr int lds =
+        (2 * LM_ROWS * LD + V * LK + 2 * LM_ROWS * LK + 2 * V * LD) * 2;
+    static bool set = false;
+    if (!set) {
+      (void)hipFuncSetAttribute(
+          reinterpret_cast<const void*>(lightning_out_mfma_kernel<D, V>),
+          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      set = true;
+    }
+    hipLaunchKernelGGL((lightning_out_mfma_kernel<D, V>), grid, block, lds,
+                       stream, out, part, (const bf16*)q, (const bf16*)k,
+                       (const bf16*)v, ldq, ldk, ldv, decay, cu, H);
+  }
+}
+
+// pass 1: part <- chunk end states; pass 2: out <- rows, part = start states.
+// Returns 1 when no kernel is built for (D, V).
+extern "C" int arks_seq_lightning_mfma(void* out, void* part, const void* q,
+                                       const void* k, const void* v,
+                                       int64_t ldq, int64_t ldk, int64_t ldv,
+                                       const void* decay, const void* cu,
+                                       int chunks, int H, int D, int V,
+                                       int pass, hipStream_t stream) {
+  if (chunks == 0) return 0;
+#define LM(DD, VV)                                                          \
+  if (D == DD && V == VV) {                                                 \
+    launch_lm<DD, VV>((float*)out, (float*)part, q, k, v, ldq, ldk, ldv,    \
+                      (const float*)decay, (const int*)cu, chunks, H, pass, \
+                      stream);                                              \
+    return 0;                                                               \
+  }
+  LM(32, 32)
+  LM(64, 64)
+  LM(128, 128)
+  LM(64, 128)
+  LM(128, 64)
+#undef LM
+  return 1;
+}

@@ -275,8 +275,9 @@ def test_long_portions_cross_the_recurrent_chunks(tmp_path, device, dtype):
     """Portions longer than one chunk of the chunk-parallel recurrent
     prefill (64 rows): one row more, exact multiples, one row less, beside
     a second request and single tokens."""
-    w = write_checkpoint(tmp_path / "m", MIXED, seed=4)
-    orc = Oracle(MIXED, w)
+    cfg = model_cfg(MIXED["layers"] + [lightning(heads=2, dim=32, vdim=32, decay=(0.95, 1.0))])
+    w = write_checkpoint(tmp_path / "m", cfg, seed=4)
+    orc = Oracle(cfg, w)
     ta, tb = toks(330, seed=31), toks(200, seed=32)
     eng = make_engine(tmp_path / "m", device, dtype, max_tokens=576)
     cuts_a = [65, 128, 1, 63, 73]

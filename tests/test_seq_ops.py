@@ -279,3 +279,38 @@ def test_chunk_parallel_scans_equal_row_by_row(dtype, lens):
     for y, st in outs[1:]:
         assert torch.allclose(y, outs[0][0], rtol=tol, atol=tol)
         assert torch.allclose(st, outs[0][1], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D,V", [(32, 32), (64, 128), (128, 128)])
+def test_lightning_matrix_core_prefill_equals_general_kernel(D, V):
+    """bf16 rows, head sizes the matrix-core kernels are built for: chunk
+    ends of 1, 63, 64 and 65 rows, decays 1, 0 and in between, old state."""
+    dev = "cuda"
+    torch.manual_seed(D + V)
+    lens = [65, 129, 200, 64]
+    T, H = sum(lens), 4
+    cu = [0]
+    for n in lens:
+        cu.append(cu[-1] + n)
+    starts = [0, 9, 500, 0]
+    meta = (i32(cu, dev), i32([s + n for s, n in zip(starts, lens)], dev),
+            i32([1, 3, 0, 2], dev))
+    chunks = ops.scan_chunks(lens, torch.device(dev))
+    q, k, v = (torch.randn(T, H, n, device=dev).to(torch.bfloat16) for n in (D, D, V))
+    decay = torch.tensor([1.0, 0.0, 0.9, 0.999], device=dev)
+    st0 = torch.randn(4, H, D, V, device=dev)
+    res = {}
+    for flag in (False, True):
+        ops.use_lightning_mfma = flag
+        try:
+            st = st0.clone()
+            o = ops.lightning_scan(q, k, v, decay, st, *meta, max_q_len=max(lens),
+                                   chunks=chunks)
+        finally:
+            ops.use_lightning_mfma = True
+        res[flag] = (o, st)
+    scale = res[False][0].abs().max()
+    assert (res[True][0] - res[False][0]).abs().max() < 1e-2 * scale
+    sscale = res[False][1].abs().max()
+    assert (res[True][1] - res[False][1]).abs().max() < 1e-2 * sscale
