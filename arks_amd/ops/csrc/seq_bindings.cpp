@@ -21,14 +21,14 @@ void arks_seq_rms_norm_f32(void* out, const void* x, const void* w,
                            int W, int act_f32, hipStream_t stream);
 void arks_seq_gelu_tanh(void* out, const void* x, int64_t ldx, int64_t rows,
                         int n, int act_f32, hipStream_t stream);
-void arks_seq_qk_norm_rope_cache(
+int arks_seq_qk_norm_rope_cache(
     void* qo, const void* q, const void* k, const void* v, int64_t ldq,
     int64_t ldk, int64_t ldv, const void* qw, const void* kw, float eps,
     const void* positions, const void* freq_qk, int n_rot, const void* freq_v,
     int n_vrot, void* k_cache, void* v_cache, const void* slot_mapping, int T,
     int H, int G, int D, int V, int block_size, int interleaved, int act_f32,
     hipStream_t stream);
-void arks_seq_unrotate_rows(void* out, const void* positions, const void* freq,
+int arks_seq_unrotate_rows(void* out, const void* positions, const void* freq,
                             int T, int H, int V, int interleaved, int act_f32,
                             hipStream_t stream);
 int arks_seq_attn_sink_generic(
@@ -275,13 +275,14 @@ void qk_norm_rope_cache(Tensor qo, Tensor q, Tensor k, Tensor v, OptTensor qw,
     TORCH_CHECK(2 * n_vrot == V, "value rotation covers all value dims");
     fv_p = freq_v->data_ptr();
   }
-  arks_seq_qk_norm_rope_cache(
+  const int rc = arks_seq_qk_norm_rope_cache(
       qo.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
       head_row_stride(q, "q"), head_row_stride(k, "k"), head_row_stride(v, "v"),
       qw_p, kw_p, (float)eps, positions.data_ptr(), freq_qk.data_ptr(), n_rot,
       fv_p, n_vrot, k_cache.data_ptr(), v_cache.data_ptr(),
       slot_mapping.data_ptr(), T, H, G, D, V, (int)k_cache.size(2),
       interleaved ? 1 : 0, f32, current_stream());
+  TORCH_CHECK(rc == 0, "more rotary pairs than the kernel's table holds");
 }
 
 void attention_sink_paged(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
@@ -329,10 +330,10 @@ void unrotate_rows(Tensor out, Tensor positions, Tensor freq_v,
   check_f32(freq_v, "inv_freq_v");
   TORCH_CHECK(positions.numel() == out.size(0) &&
               2 * freq_v.numel() == out.size(2));
-  arks_seq_unrotate_rows(out.data_ptr(), positions.data_ptr(),
-                         freq_v.data_ptr(), out.size(0), out.size(1),
-                         out.size(2), interleaved ? 1 : 0, f32,
-                         current_stream());
+  const int rc = arks_seq_unrotate_rows(
+      out.data_ptr(), positions.data_ptr(), freq_v.data_ptr(), out.size(0),
+      out.size(1), out.size(2), interleaved ? 1 : 0, f32, current_stream());
+  TORCH_CHECK(rc == 0, "more rotary pairs than the kernel's table holds");
 }
 
 void lightning_scan(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,

@@ -197,13 +197,38 @@ __global__ __launch_bounds__(256) void gelu_tanh_kernel(
   Act<AT>::st(out + idx, 0.5f * z * (1.f + tanhf(u)));
 }
 
-// One wave per (row, head slot): slots [0,H) are query heads, [H,H+G) key
-// heads, [H+G,H+2G) value heads. q/k: RMS norm over the head (weight or
-// none) then rotary on the first 2*n_rot dims; v: turned by the row's
-// position over all its dims (n_vrot pairs; 0 = stored plain). Pairs are
-// (2i,2i+1) when interleaved, (i, i+n) otherwise. k and v go to their page.
+// bf16, 8 elements per thread; tanh(u) = 1 - 2 / (1 + e^(2u)) with the
+// hardware exponential (saturates cleanly at both ends)
+__global__ __launch_bounds__(256) void gelu_tanh_vec8_kernel(
+    bf16* __restrict__ out, const bf16* __restrict__ x, int64_t ldx,
+    int64_t rows, int n8) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * n8) return;
+  const int64_t r = idx / n8;
+  const int c = (int)(idx - r * n8) * 8;
+  const ushort8 v = *reinterpret_cast<const ushort8*>(x + r * ldx + c);
+  ushort8 o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float z = bf16_bits_to_float(v[e]);
+    const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+    const float th = 1.f - 2.f / (1.f + __expf(2.f * u));
+    o[e] = float_to_bf16_bits(0.5f * z * (1.f + th));
+  }
+  *reinterpret_cast<ushort8*>(out + r * (int64_t)n8 * 8 + c) = o;
+}
+
+// One block per row: the row's rotary angles (they depend on the position
+// and the pair only) are evaluated once into LDS, then the block's waves
+// walk the head slots — [0,H) query heads, [H,H+G) key heads, [H+G,H+2G)
+// value heads. q/k: RMS norm over the head (weight or none) then rotary on
+// the first 2*n_rot dims; v: turned by the row's position over all its dims
+// (n_vrot pairs; 0 = stored plain). Pairs are (2i,2i+1) when interleaved,
+// (i, i+n) otherwise. k and v go to their page.
+constexpr int ROPE_MAX_PAIRS = 256;
+
 template <typename AT>
-__global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
+__global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
     AT* __restrict__ qo, const AT* __restrict__ q, const AT* __restrict__ k,
     const AT* __restrict__ v, int64_t ldq, int64_t ldk, int64_t ldv,
     const float* __restrict__ qw, const float* __restrict__ kw, float eps,
@@ -212,83 +237,94 @@ __global__ __launch_bounds__(64) void qk_norm_rope_cache_kernel(
     AT* __restrict__ k_cache, AT* __restrict__ v_cache,
     const int64_t* __restrict__ slot_mapping, int H, int G, int D, int V,
     int block_size, int interleaved) {
+  __shared__ float cs_qk[ROPE_MAX_PAIRS][2];
+  __shared__ float cs_v[ROPE_MAX_PAIRS][2];
   const int t = blockIdx.x;
-  const int hs = blockIdx.y;
-  const int lane = threadIdx.x;
   const float pos = (float)positions[t];
-  const AT* src;
-  AT* dst;
-  const float* nw = nullptr;
-  const float* freq;
-  int n, npairs;
-  bool normed;
-  if (hs < H) {
-    src = q + (int64_t)t * ldq + (int64_t)hs * D;
-    dst = qo + ((int64_t)t * H + hs) * D;
-    n = D; npairs = n_rot; freq = freq_qk; nw = qw; normed = qw != nullptr;
-  } else {
-    const int64_t slot = slot_mapping[t];
-    if (slot < 0) return;
-    const int64_t blk = slot / block_size, off = slot % block_size;
-    if (hs < H + G) {
-      const int g = hs - H;
-      src = k + (int64_t)t * ldk + (int64_t)g * D;
-      dst = k_cache + ((blk * G + g) * block_size + off) * D;
-      n = D; npairs = n_rot; freq = freq_qk; nw = kw; normed = kw != nullptr;
+  for (int i = threadIdx.x; i < n_rot; i += 256)
+    sincosf(pos * freq_qk[i], &cs_qk[i][1], &cs_qk[i][0]);
+  for (int i = threadIdx.x; i < n_vrot; i += 256)
+    sincosf(pos * freq_v[i], &cs_v[i][1], &cs_v[i][0]);
+  __syncthreads();
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int64_t slot = slot_mapping[t];
+  for (int hs = wave; hs < H + 2 * G; hs += 4) {
+    const AT* src;
+    AT* dst;
+    const float* nw = nullptr;
+    const float(*cs)[2];
+    int n, npairs;
+    if (hs < H) {
+      src = q + (int64_t)t * ldq + (int64_t)hs * D;
+      dst = qo + ((int64_t)t * H + hs) * D;
+      n = D; npairs = n_rot; cs = cs_qk; nw = qw;
     } else {
-      const int g = hs - H - G;
-      src = v + (int64_t)t * ldv + (int64_t)g * V;
-      dst = v_cache + ((blk * G + g) * block_size + off) * V;
-      n = V; npairs = n_vrot; freq = freq_v; normed = false;
+      if (slot < 0) continue;
+      const int64_t blk = slot / block_size, off = slot % block_size;
+      if (hs < H + G) {
+        const int g = hs - H;
+        src = k + (int64_t)t * ldk + (int64_t)g * D;
+        dst = k_cache + ((blk * G + g) * block_size + off) * D;
+        n = D; npairs = n_rot; cs = cs_qk; nw = kw;
+      } else {
+        const int g = hs - H - G;
+        src = v + (int64_t)t * ldv + (int64_t)g * V;
+        dst = v_cache + ((blk * G + g) * block_size + off) * V;
+        n = V; npairs = n_vrot; cs = cs_v;
+      }
     }
-  }
-  float rstd = 1.f;
-  if (normed) {
-    float ss = 0.f;
-    for (int i = lane; i < n; i += 64) {
-      const float a = Act<AT>::ld(src + i);
-      ss += a * a;
+    const bool normed = nw != nullptr;
+    float rstd = 1.f;
+    if (normed) {
+      float ss = 0.f;
+      for (int i = lane; i < n; i += 64) {
+        const float a = Act<AT>::ld(src + i);
+        ss += a * a;
+      }
+      ss = wave_reduce_sum(ss);
+      rstd = 1.f / sqrtf(ss / (float)n + eps);
     }
-    ss = wave_reduce_sum(ss);
-    rstd = 1.f / sqrtf(ss / (float)n + eps);
-  }
-  for (int i = lane; i < npairs; i += 64) {
-    const int d0 = interleaved ? 2 * i : i;
-    const int d1 = interleaved ? 2 * i + 1 : i + npairs;
-    float a = Act<AT>::ld(src + d0) * rstd;
-    float b = Act<AT>::ld(src + d1) * rstd;
-    if (normed) { a *= nw[d0]; b *= nw[d1]; }
-    float sn, cs;
-    sincosf(pos * freq[i], &sn, &cs);
-    Act<AT>::st(dst + d0, a * cs - b * sn);
-    Act<AT>::st(dst + d1, b * cs + a * sn);
-  }
-  for (int i = 2 * npairs + lane; i < n; i += 64) {
-    float a = Act<AT>::ld(src + i) * rstd;
-    if (normed) a *= nw[i];
-    Act<AT>::st(dst + i, a);
+    for (int i = lane; i < npairs; i += 64) {
+      const int d0 = interleaved ? 2 * i : i;
+      const int d1 = interleaved ? 2 * i + 1 : i + npairs;
+      float a = Act<AT>::ld(src + d0) * rstd;
+      float b = Act<AT>::ld(src + d1) * rstd;
+      if (normed) { a *= nw[d0]; b *= nw[d1]; }
+      const float c = cs[i][0], sn = cs[i][1];
+      Act<AT>::st(dst + d0, a * c - b * sn);
+      Act<AT>::st(dst + d1, b * c + a * sn);
+    }
+    for (int i = 2 * npairs + lane; i < n; i += 64) {
+      float a = Act<AT>::ld(src + i) * rstd;
+      if (normed) a *= nw[i];
+      Act<AT>::st(dst + i, a);
+    }
   }
 }
 
 // Turn every head row of out [T, H, V] back by its row's position: pair m
 // by -pos * freq[m] (the cache holds values turned forward by their own
-// positions, so the weighted sum comes out in the query's frame).
+// positions, so the weighted sum comes out in the query's frame). One block
+// per row, the angles evaluated once for all heads.
 template <typename AT>
-__global__ __launch_bounds__(64) void unrotate_rows_kernel(
+__global__ __launch_bounds__(256) void unrotate_rows_kernel(
     AT* __restrict__ out, const int64_t* __restrict__ positions,
-    const float* __restrict__ freq, int V, int interleaved) {
-  const int t = blockIdx.x, h = blockIdx.y;
-  AT* row = out + ((int64_t)t * gridDim.y + h) * V;
+    const float* __restrict__ freq, int H, int V, int interleaved) {
+  __shared__ float cs[ROPE_MAX_PAIRS][2];
+  const int t = blockIdx.x;
   const float pos = (float)positions[t];
   const int npairs = V / 2;
-  for (int i = threadIdx.x; i < npairs; i += 64) {
+  for (int i = threadIdx.x; i < npairs; i += 256)
+    sincosf(-pos * freq[i], &cs[i][1], &cs[i][0]);
+  __syncthreads();
+  for (int e = threadIdx.x; e < H * npairs; e += 256) {
+    const int h = e / npairs, i = e - h * npairs;
+    AT* row = out + ((int64_t)t * H + h) * V;
     const int d0 = interleaved ? 2 * i : i;
     const int d1 = interleaved ? 2 * i + 1 : i + npairs;
     const float a = Act<AT>::ld(row + d0), b = Act<AT>::ld(row + d1);
-    float sn, cs;
-    sincosf(-pos * freq[i], &sn, &cs);
-    Act<AT>::st(row + d0, a * cs - b * sn);
-    Act<AT>::st(row + d1, b * cs + a * sn);
+    Act<AT>::st(row + d0, a * cs[i][0] - b * cs[i][1]);
+    Act<AT>::st(row + d1, b * cs[i][0] + a * cs[i][1]);
   }
 }
 
@@ -296,14 +332,16 @@ __global__ __launch_bounds__(64) void unrotate_rows_kernel(
 
 using namespace arks;
 
-extern "C" void arks_seq_unrotate_rows(void* out, const void* positions,
-                                       const void* freq, int T, int H, int V,
-                                       int interleaved, int act_f32,
-                                       hipStream_t stream) {
-  if (T == 0) return;
+extern "C" int arks_seq_unrotate_rows(void* out, const void* positions,
+                                      const void* freq, int T, int H, int V,
+                                      int interleaved, int act_f32,
+                                      hipStream_t stream) {
+  if (V / 2 > ROPE_MAX_PAIRS) return 1;
+  if (T == 0) return 0;
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
-      (unrotate_rows_kernel<AT>), dim3(T, H), dim3(64), 0, stream, (AT*)out,
-      (const int64_t*)positions, (const float*)freq, V, interleaved));
+      (unrotate_rows_kernel<AT>), dim3(T), dim3(256), 0, stream, (AT*)out,
+      (const int64_t*)positions, (const float*)freq, H, V, interleaved));
+  return 0;
 }
 
 extern "C" void arks_seq_token_shift(void* xs, void* xa, const void* x,
@@ -360,24 +398,32 @@ extern "C" void arks_seq_gelu_tanh(void* out, const void* x, int64_t ldx,
                                    hipStream_t stream) {
   const int64_t total = rows * n;
   if (total == 0) return;
+  if (!act_f32 && n % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0) {
+    hipLaunchKernelGGL(gelu_tanh_vec8_kernel,
+                       dim3((unsigned)((total / 8 + 255) / 256)), dim3(256), 0,
+                       stream, (bf16*)out, (const bf16*)x, ldx, rows, n / 8);
+    return;
+  }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (gelu_tanh_kernel<AT>), dim3((unsigned)((total + 255) / 256)), dim3(256),
       0, stream, (AT*)out, (const AT*)x, ldx, rows, n));
 }
 
-extern "C" void arks_seq_qk_norm_rope_cache(
+extern "C" int arks_seq_qk_norm_rope_cache(
     void* qo, const void* q, const void* k, const void* v, int64_t ldq,
     int64_t ldk, int64_t ldv, const void* qw, const void* kw, float eps,
     const void* positions, const void* freq_qk, int n_rot, const void* freq_v,
     int n_vrot, void* k_cache, void* v_cache, const void* slot_mapping, int T,
     int H, int G, int D, int V, int block_size, int interleaved, int act_f32,
     hipStream_t stream) {
-  if (T == 0) return;
+  if (n_rot > ROPE_MAX_PAIRS || n_vrot > ROPE_MAX_PAIRS) return 1;
+  if (T == 0) return 0;
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
-      (qk_norm_rope_cache_kernel<AT>), dim3(T, H + 2 * G), dim3(64), 0, stream,
+      (qk_norm_rope_cache_kernel<AT>), dim3(T), dim3(256), 0, stream,
       (AT*)qo, (const AT*)q, (const AT*)k, (const AT*)v, ldq, ldk, ldv,
       (const float*)qw, (const float*)kw, eps, (const int64_t*)positions,
       (const float*)freq_qk, n_rot, (const float*)freq_v, n_vrot, (AT*)k_cache,
       (AT*)v_cache, (const int64_t*)slot_mapping, H, G, D, V, block_size,
       interleaved));
+  return 0;
 }
