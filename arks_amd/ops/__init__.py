@@ -754,8 +754,9 @@ def lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
             if not mfma:
                 S.lightning_scan(out, q, k, v, decay, part, c["cu"],
                                  c["lens0"], c["slots"], SCAN_CHUNK)
+            # the matrix-core passes keep their scratch states transposed
             S.lightning_combine(part, decay, state, c["off"], c["rows"],
-                                cu_seqlens, seq_lens, state_slots)
+                                cu_seqlens, seq_lens, state_slots, mfma)
             if mfma:
                 S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 2)
             else:

@@ -69,8 +69,8 @@ int arks_seq_lightning_mfma(void* out, void* part, const void* q, const void* k,
 void arks_seq_lightning_combine(void* part, const void* decay, void* state,
                                 const void* chunk_off, const void* chunk_rows,
                                 const void* cu, const void* seq_lens,
-                                const void* slots, int S, int H, int DV,
-                                hipStream_t stream);
+                                const void* slots, int S, int H, int D, int V,
+                                int transposed, hipStream_t stream);
 }
 
 namespace {
@@ -501,14 +501,15 @@ bool lightning_mfma(Tensor out, Tensor part, Tensor q, Tensor k, Tensor v,
 
 void lightning_combine(Tensor part, Tensor decay, Tensor state,
                        Tensor chunk_off, Tensor chunk_rows, Tensor cu,
-                       Tensor seq_lens, Tensor slots) {
+                       Tensor seq_lens, Tensor slots, bool transposed) {
   check_f32(part, "part");
   check_f32(decay, "decay");
   check_f32(state, "state");
+  // part: [chunks, H, D, V], or its states stored [v][d] (transposed)
   TORCH_CHECK(part.dim() == 4 && state.dim() == 4 &&
-              part.size(1) == state.size(1) && part.size(2) == state.size(2) &&
-              part.size(3) == state.size(3));
-  const int H = state.size(1), DV = state.size(2) * state.size(3);
+              part.size(1) == state.size(1) &&
+              part.size(2) * part.size(3) == state.size(2) * state.size(3));
+  const int H = state.size(1), D = state.size(2), V = state.size(3);
   TORCH_CHECK(decay.numel() == H);
   const SeqMeta m = check_meta(cu, seq_lens, &slots, nullptr, 0);
   check_i32(chunk_off, "chunk_off");
@@ -518,8 +519,8 @@ void lightning_combine(Tensor part, Tensor decay, Tensor state,
   arks_seq_lightning_combine(part.data_ptr(), decay.data_ptr(),
                              state.data_ptr(), chunk_off.data_ptr(),
                              chunk_rows.data_ptr(), cu.data_ptr(),
-                             seq_lens.data_ptr(), slots.data_ptr(), m.S, H, DV,
-                             current_stream());
+                             seq_lens.data_ptr(), slots.data_ptr(), m.S, H, D,
+                             V, transposed ? 1 : 0, current_stream());
 }
 
 }  // namespace

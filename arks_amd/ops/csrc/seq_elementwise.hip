@@ -173,11 +173,30 @@ __global__ __launch_bounds__(256) void rms_norm_f32_kernel(
   __shared__ float scratch[4];
   const int t = blockIdx.x;
   const float* xr = x + (int64_t)t * W;
+  // the first 16 * 256 elements of the row stay in registers between the
+  // two passes; longer rows re-read their tail
+  constexpr int KEEP = 16;
+  float xv[KEEP];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < W; i += 256) ss += xr[i] * xr[i];
+#pragma unroll
+  for (int u = 0; u < KEEP; ++u) {
+    const int i = threadIdx.x + 256 * u;
+    xv[u] = i < W ? xr[i] : 0.f;
+    ss += xv[u] * xv[u];
+  }
+  for (int i = threadIdx.x + 256 * KEEP; i < W; i += 256) ss += xr[i] * xr[i];
   ss = block_reduce_sum<256>(ss, scratch);
   const float rstd = 1.f / sqrtf(ss / (float)W + eps);
-  for (int i = threadIdx.x; i < W; i += 256) {
+#pragma unroll
+  for (int u = 0; u < KEEP; ++u) {
+    const int i = threadIdx.x + 256 * u;
+    if (i < W) {
+      float v = xv[u] * rstd * w[i];
+      if (gate) v *= sigmoid_f(Act<AT>::ld(gate + (int64_t)t * ldg + i));
+      Act<AT>::st(out + (int64_t)t * W + i, v);
+    }
+  }
+  for (int i = threadIdx.x + 256 * KEEP; i < W; i += 256) {
     float v = xr[i] * rstd * w[i];
     if (gate) v *= sigmoid_f(Act<AT>::ld(gate + (int64_t)t * ldg + i));
     Act<AT>::st(out + (int64_t)t * W + i, v);
@@ -274,25 +293,40 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(
       }
     }
     const bool normed = nw != nullptr;
+    // the head is read once: this lane's pairs stay in registers between
+    // the sum of squares and the rotation (npairs <= 64 * 4)
+    float pa[ROPE_MAX_PAIRS / 64], pb[ROPE_MAX_PAIRS / 64];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < ROPE_MAX_PAIRS / 64; ++u) {
+      const int i = lane + 64 * u;
+      if (i < npairs) {
+        pa[u] = Act<AT>::ld(src + (interleaved ? 2 * i : i));
+        pb[u] = Act<AT>::ld(src + (interleaved ? 2 * i + 1 : i + npairs));
+        ss += pa[u] * pa[u] + pb[u] * pb[u];
+      }
+    }
     float rstd = 1.f;
     if (normed) {
-      float ss = 0.f;
-      for (int i = lane; i < n; i += 64) {
+      for (int i = 2 * npairs + lane; i < n; i += 64) {
         const float a = Act<AT>::ld(src + i);
         ss += a * a;
       }
       ss = wave_reduce_sum(ss);
       rstd = 1.f / sqrtf(ss / (float)n + eps);
     }
-    for (int i = lane; i < npairs; i += 64) {
-      const int d0 = interleaved ? 2 * i : i;
-      const int d1 = interleaved ? 2 * i + 1 : i + npairs;
-      float a = Act<AT>::ld(src + d0) * rstd;
-      float b = Act<AT>::ld(src + d1) * rstd;
-      if (normed) { a *= nw[d0]; b *= nw[d1]; }
-      const float c = cs[i][0], sn = cs[i][1];
-      Act<AT>::st(dst + d0, a * c - b * sn);
-      Act<AT>::st(dst + d1, b * c + a * sn);
+#pragma unroll
+    for (int u = 0; u < ROPE_MAX_PAIRS / 64; ++u) {
+      const int i = lane + 64 * u;
+      if (i < npairs) {
+        const int d0 = interleaved ? 2 * i : i;
+        const int d1 = interleaved ? 2 * i + 1 : i + npairs;
+        float a = pa[u] * rstd, b = pb[u] * rstd;
+        if (normed) { a *= nw[d0]; b *= nw[d1]; }
+        const float c = cs[i][0], sn = cs[i][1];
+        Act<AT>::st(dst + d0, a * c - b * sn);
+        Act<AT>::st(dst + d1, b * c + a * sn);
+      }
     }
     for (int i = 2 * npairs + lane; i < n; i += 64) {
       float a = Act<AT>::ld(src + i) * rstd;

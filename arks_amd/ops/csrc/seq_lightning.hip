@@ -69,23 +69,30 @@ __global__ __launch_bounds__(256) void lightning_combine_kernel(
     float* __restrict__ state, const int* __restrict__ chunk_off,
     const int* __restrict__ chunk_rows, const int* __restrict__ cu,
     const int* __restrict__ seq_lens, const int* __restrict__ slots, int H,
-    int DV) {
+    int D, int V, int transposed) {
+  const int DV = D * V;
   const int s = blockIdx.y;
   const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (e >= (int64_t)H * DV) return;
+  // the scratch states may be stored [v][d]; the slot state is [d][v]
+  int64_t se = e;
+  if (transposed) {
+    const int hh = (int)(e / DV), rem = (int)(e - (int64_t)hh * DV);
+    se = (int64_t)hh * DV + (int64_t)(rem % D) * V + rem / D;
+  }
   const int rows = cu[s + 1] - cu[s];
   if (rows == 0) return;
   const int start = seq_lens[s] - rows;
   const int slot = slots[s];
   const float lam = decay[e / DV];
-  float carry = (start > 0 && slot >= 0) ? state[(int64_t)slot * H * DV + e] : 0.f;
+  float carry = (start > 0 && slot >= 0) ? state[(int64_t)slot * H * DV + se] : 0.f;
   for (int k = chunk_off[s]; k < chunk_off[s + 1]; ++k) {
     float* p = part + (int64_t)k * H * DV + e;
     const float local = *p;
     *p = carry;
     carry = powf(lam, (float)chunk_rows[k]) * carry + local;
   }
-  if (slot >= 0) state[(int64_t)slot * H * DV + e] = carry;
+  if (slot >= 0) state[(int64_t)slot * H * DV + se] = carry;
 }
 
 }  // namespace arks
@@ -97,15 +104,16 @@ extern "C" void arks_seq_lightning_combine(void* part, const void* decay,
                                            const void* chunk_rows,
                                            const void* cu, const void* seq_lens,
                                            const void* slots, int S, int H,
-                                           int DV, hipStream_t stream) {
+                                           int D, int V, int transposed,
+                                           hipStream_t stream) {
   if (S == 0) return;
-  const int64_t n = (int64_t)H * DV;
+  const int64_t n = (int64_t)H * D * V;
   hipLaunchKernelGGL(lightning_combine_kernel,
                      dim3((unsigned)((n + 255) / 256), S), dim3(256), 0, stream,
                      (float*)part, (const float*)decay, (float*)state,
                      (const int*)chunk_off, (const int*)chunk_rows,
                      (const int*)cu, (const int*)seq_lens, (const int*)slots, H,
-                     DV);
+                     D, V, transposed);
 }
 
 template <typename AT>

@@ -6,6 +6,9 @@
 //   pass 2  o_i = decay^(i+1) (q_i . S0) + sum_{j<=i} decay^(i-j) (q_i.k_j) v_j
 //
 // with S0 the chunk's start state left in `part` by lightning_combine.
+// `part` holds each state TRANSPOSED ([v][d]): pass 2 then reads its state
+// operand (k = d contiguous) straight from global memory, and the combine
+// step between the passes is elementwise, so it does not care.
 // q, k, v are silu'd in fp32 on the way into LDS and rounded to bf16 for
 // v_mfma_f32_16x16x32_bf16. Every fp32 quantity that meets a matrix
 // operand — the decayed keys of pass 1, the decayed score matrix and the
@@ -37,6 +40,14 @@ __device__ __forceinline__ lm_f32x4 lm_mfma(const bf16* a, const bf16* b,
       0, 0, 0);
 }
 
+__device__ __forceinline__ lm_f32x4 lm_mfma_r(const bf16* a, ushort8 ub,
+                                              lm_f32x4 c) {
+  ushort8 ua = *reinterpret_cast<const ushort8*>(a);
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+      *reinterpret_cast<lm_bf16x8*>(&ua), *reinterpret_cast<lm_bf16x8*>(&ub), c,
+      0, 0, 0);
+}
+
 __device__ __forceinline__ void split_bf16(float x, bf16& hi, bf16& lo) {
   hi = float_to_bf16_bits(x);
   lo = float_to_bf16_bits(x - bf16_bits_to_float(hi));
@@ -50,7 +61,7 @@ __device__ __forceinline__ float decay_pow(float log2_decay, int e) {
 // ---- pass 1: end state of each chunk scanned from zero
 template <int D, int V>
 __global__ __launch_bounds__(256) void lightning_state_mfma_kernel(
-    float* __restrict__ part,  // [chunks, H, D, V]
+    float* __restrict__ part,  // [chunks, H, V, D] (transposed states)
     const bf16* __restrict__ k, const bf16* __restrict__ v, int64_t ldk,
     int64_t ldv, const float* __restrict__ decay, const int* __restrict__ cu,
     int H) {
@@ -89,20 +100,21 @@ __global__ __launch_bounds__(256) void lightning_state_mfma_kernel(
 #pragma unroll
     for (int st = 0; st < LM_ROWS / 32; ++st) {
       const int ko = st * 32 + 8 * la;
-      const bf16* ah = kt_hi + (dt * 16 + lq) * LK + ko;
-      const bf16* al = kt_lo + (dt * 16 + lq) * LK + ko;
+      const bf16* bh = kt_hi + (dt * 16 + lq) * LK + ko;
+      const bf16* bl = kt_lo + (dt * 16 + lq) * LK + ko;
 #pragma unroll
       for (int c = 0; c < VT; ++c) {
-        const bf16* b = vt + (c * 16 + lq) * LK + ko;
-        acc[c] = lm_mfma(ah, b, acc[c]);
-        acc[c] = lm_mfma(al, b, acc[c]);
+        const bf16* a = vt + (c * 16 + lq) * LK + ko;  // rows = value dims
+        acc[c] = lm_mfma(a, bh, acc[c]);
+        acc[c] = lm_mfma(a, bl, acc[c]);
       }
     }
+    // result rows m = value dim, column n = key dim: out[v][d]
 #pragma unroll
     for (int c = 0; c < VT; ++c)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        out[(int64_t)(dt * 16 + 4 * la + r) * V + c * 16 + lq] = acc[c][r];
+        out[(int64_t)(c * 16 + 4 * la + r) * D + dt * 16 + lq] = acc[c][r];
   }
 }
 
@@ -110,7 +122,7 @@ __global__ __launch_bounds__(256) void lightning_state_mfma_kernel(
 template <int D, int V>
 __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
     float* __restrict__ out,         // [T, H, V] fp32
-    const float* __restrict__ part,  // [chunks, H, D, V] start states
+    const float* __restrict__ part,  // [chunks, H, V, D] start states^T
     const bf16* __restrict__ q, const bf16* __restrict__ k,
     const bf16* __restrict__ v, int64_t ldq, int64_t ldk, int64_t ldv,
     const float* __restrict__ decay, const int* __restrict__ cu, int H) {
@@ -122,8 +134,6 @@ __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
   bf16* vt = ks + LM_ROWS * LD;                 // [V][LK]
   bf16* a_hi = vt + V * LK;                     // [64][LK]
   bf16* a_lo = a_hi + LM_ROWS * LK;             // [64][LK]
-  bf16* st_hi = a_lo + LM_ROWS * LK;            // [V][LD]  state^T
-  bf16* st_lo = st_hi + V * LD;                 // [V][LD]
   const int ch = blockIdx.x, h = blockIdx.y;
   const int row0 = cu[ch], n = cu[ch + 1] - row0;
   const float l2 = log2f(decay[h]);
@@ -145,13 +155,7 @@ __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
       x = silu_f(bf16_bits_to_float(v[(int64_t)(row0 + j) * ldv + (int64_t)h * V + c]));
     vt[c * LK + j] = float_to_bf16_bits(x);
   }
-  {
-    const float* sp = part + ((int64_t)ch * H + h) * D * V;
-    for (int i = tid; i < D * V; i += 256) {
-      const int d = i / V, c = i - d * V;
-      split_bf16(sp[i], st_hi[c * LD + d], st_lo[c * LD + d]);
-    }
-  }
+  const float* sp = part + ((int64_t)ch * H + h) * D * V;  // [V][D]
   __syncthreads();
   const int wave = tid / 64, lane = tid % 64, lq = lane % 16, la = lane / 16;
   // scores of this wave's 16 rows against all 64 keys, decayed and masked,
@@ -196,8 +200,20 @@ __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
     const int ko = st * 32 + 8 * la;
 #pragma unroll
     for (int c = 0; c < VT; ++c) {
-      acs[c] = lm_mfma(qs + arow * LD + ko, st_hi + (c * 16 + lq) * LD + ko, acs[c]);
-      acs[c] = lm_mfma(qs + arow * LD + ko, st_lo + (c * 16 + lq) * LD + ko, acs[c]);
+      // 8 consecutive key dims of state row v = 16 c + lq, fp32 -> hi + lo
+      const float* sr = sp + (int64_t)(c * 16 + lq) * D + ko;
+      const float4v s0 = *reinterpret_cast<const float4v*>(sr);
+      const float4v s1 = *reinterpret_cast<const float4v*>(sr + 4);
+      ushort8 bh, bl;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        bf16 h0, l0, h1, l1;
+        split_bf16(s0[e], h0, l0);
+        split_bf16(s1[e], h1, l1);
+        bh[e] = h0; bl[e] = l0; bh[4 + e] = h1; bl[4 + e] = l1;
+      }
+      acs[c] = lm_mfma_r(qs + arow * LD + ko, bh, acs[c]);
+      acs[c] = lm_mfma_r(qs + arow * LD + ko, bl, acs[c]);
     }
   }
 #pragma unroll
@@ -235,8 +251,7 @@ static void launch_lm(float* out, float* part, const void* q, const void* k,
                        stream, part, (const bf16*)k, (const bf16*)v, ldk, ldv,
                        decay, cu, H);
   } else {
-    constexpr int lds =
-        (2 * LM_ROWS * LD + V * LK + 2 * LM_ROWS * LK + 2 * V * LD) * 2;
+    constexpr int lds = (2 * LM_ROWS * LD + V * LK + 2 * LM_ROWS * LK) * 2;
     static bool set = false;
     if (!set) {
       (void)hipFuncSetAttribute(

@@ -41,58 +41,78 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
   }
 }
 
-// bf16 rows, 8 channels per thread: 16-byte loads of each tap's row, conv
-// taps from a transposed copy of the weights (w_t [taps, C]) so that they
-// load as two float4 per tap.
+// bf16 rows, 8 channels per thread and CONV_RPT consecutive rows per block:
+// 16-byte loads of each tap's row, the conv taps of the thread's channels
+// held in registers across the rows (w_t [taps, C] is a transposed copy of
+// the weights so that they load as two float4 per tap).
+constexpr int CONV_RPT = 8;
+constexpr int CONV_MAX_TAPS = CONV_MAX_HIST + 1;
+
 __global__ __launch_bounds__(256) void causal_conv_silu_vec8_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ x, int64_t ldx,
     const float* __restrict__ w_t, const float* __restrict__ bias,
     const float* __restrict__ state, const int* __restrict__ cu,
     const int* __restrict__ seq_lens, const int* __restrict__ slots,
-    const int* __restrict__ token_seq, int C, int taps) {
-  const int t = blockIdx.x;
+    const int* __restrict__ token_seq, int T, int C, int taps) {
   const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
   if (c >= C) return;
-  const SeqRow r = seq_row(t, token_seq, cu, seq_lens, slots);
-  const int i = t - r.first_row;
-  const bool has_state = r.start > 0 && r.slot >= 0;
-  const float* hist = state + (int64_t)(r.slot < 0 ? 0 : r.slot) * (taps - 1) * C;
-  float acc[8];
+  float wv[CONV_MAX_TAPS][8], bv[8];
   {
     const float4v b0 = *reinterpret_cast<const float4v*>(bias + c);
     const float4v b1 = *reinterpret_cast<const float4v*>(bias + c + 4);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) { acc[e] = b0[e]; acc[4 + e] = b1[e]; }
+    for (int e = 0; e < 4; ++e) { bv[e] = b0[e]; bv[4 + e] = b1[e]; }
   }
-  for (int j = 0; j < taps; ++j) {
-    const int src = i - (taps - 1 - j);
-    float xv[8];
-    if (src >= 0) {
-      const ushort8 v = *reinterpret_cast<const ushort8*>(
-          x + (int64_t)(r.first_row + src) * ldx + c);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) xv[e] = bf16_bits_to_float(v[e]);
-    } else if (has_state) {
-      const float* hp = hist + (int64_t)(src + taps - 1) * C + c;
-      const float4v h0 = *reinterpret_cast<const float4v*>(hp);
-      const float4v h1 = *reinterpret_cast<const float4v*>(hp + 4);
+  for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+    if (j < taps) {
+      const float4v w0 = *reinterpret_cast<const float4v*>(w_t + (int64_t)j * C + c);
+      const float4v w1 = *reinterpret_cast<const float4v*>(w_t + (int64_t)j * C + c + 4);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) { xv[e] = h0[e]; xv[4 + e] = h1[e]; }
-    } else {
-      continue;
-    }
-    const float4v w0 = *reinterpret_cast<const float4v*>(w_t + (int64_t)j * C + c);
-    const float4v w1 = *reinterpret_cast<const float4v*>(w_t + (int64_t)j * C + c + 4);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      acc[e] += w0[e] * xv[e];
-      acc[4 + e] += w1[e] * xv[4 + e];
+      for (int e = 0; e < 4; ++e) { wv[j][e] = w0[e]; wv[j][4 + e] = w1[e]; }
     }
   }
-  ushort8 o;
+  const int t_end = min(T, (int)(blockIdx.x + 1) * CONV_RPT);
+  for (int t = blockIdx.x * CONV_RPT; t < t_end; ++t) {
+    const SeqRow r = seq_row(t, token_seq, cu, seq_lens, slots);
+    const int i = t - r.first_row;
+    const bool has_state = r.start > 0 && r.slot >= 0;
+    const float* hist =
+        state + (int64_t)(r.slot < 0 ? 0 : r.slot) * (taps - 1) * C;
+    float acc[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = float_to_bf16_bits(silu_f(acc[e]));
-  *reinterpret_cast<ushort8*>(out + (int64_t)t * C + c) = o;
+    for (int e = 0; e < 8; ++e) acc[e] = bv[e];
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+      if (j < taps) {
+        const int src = i - (taps - 1 - j);
+        float xv[8];
+        bool have = true;
+        if (src >= 0) {
+          const ushort8 v = *reinterpret_cast<const ushort8*>(
+              x + (int64_t)(r.first_row + src) * ldx + c);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) xv[e] = bf16_bits_to_float(v[e]);
+        } else if (has_state) {
+          const float* hp = hist + (int64_t)(src + taps - 1) * C + c;
+          const float4v h0 = *reinterpret_cast<const float4v*>(hp);
+          const float4v h1 = *reinterpret_cast<const float4v*>(hp + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { xv[e] = h0[e]; xv[4 + e] = h1[e]; }
+        } else {
+          have = false;
+        }
+        if (have) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] += wv[j][e] * xv[e];
+        }
+      }
+    }
+    ushort8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = float_to_bf16_bits(silu_f(acc[e]));
+    *reinterpret_cast<ushort8*>(out + (int64_t)t * C + c) = o;
+  }
 }
 
 // New history of a sequence = the last taps-1 inputs after this step: rows
@@ -335,11 +355,13 @@ extern "C" int arks_seq_causal_conv_silu(
   SEQ_DISPATCH_ACT(act_f32, {
     if (vec8)
       hipLaunchKernelGGL(causal_conv_silu_vec8_kernel,
-                         dim3(T, (C / 8 + 255) / 256), dim3(256), 0, stream,
-                         (bf16*)out, (const bf16*)x, ldx, (const float*)w_t,
-                         (const float*)bias, (const float*)state,
-                         (const int*)cu, (const int*)seq_lens,
-                         (const int*)slots, (const int*)token_seq, C, taps);
+                         dim3((T + CONV_RPT - 1) / CONV_RPT,
+                              (C / 8 + 255) / 256),
+                         dim3(256), 0, stream, (bf16*)out, (const bf16*)x, ldx,
+                         (const float*)w_t, (const float*)bias,
+                         (const float*)state, (const int*)cu,
+                         (const int*)seq_lens, (const int*)slots,
+                         (const int*)token_seq, T, C, taps);
     else
     hipLaunchKernelGGL((causal_conv_silu_kernel<AT>), dim3(T, cb), dim3(256), 0,
                        stream, (AT*)out, (const AT*)x, ldx, (const float*)w,
