@@ -36,6 +36,10 @@ def parse_args(argv=None):
                    default=None)
     p.add_argument("--quantization", choices=["fp8"], default=None)
     p.add_argument("--kv-cache-dtype", choices=["auto", "fp8"], default="auto")
+    p.add_argument("--dtype", choices=["bfloat16", "float32"],
+                   default="bfloat16",
+                   help="float32: true 32-bit serving, for the models that "
+                        "implement it (Gagorax)")
     p.add_argument("--speculative", choices=["ngram", "draft"], default=None,
                    help="speculative decoding: ngram (prompt lookup) or "
                         "draft (a smaller draft model, --draft-model)")
@@ -73,6 +77,7 @@ def build_engine_config(args):
         enforce_eager=args.enforce_eager,
         quantization=args.quantization,
         kv_cache_dtype=args.kv_cache_dtype,
+        dtype=args.dtype,
         speculative=args.speculative,
         draft_model=args.draft_model,
         num_speculative_tokens=args.num_speculative_tokens,
