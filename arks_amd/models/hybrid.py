@@ -36,7 +36,7 @@ from .. import ops
 from ..config import HybridModelConfig
 from ..engine.forward_batch import ForwardBatch
 from ..parallel.comm import get_tp_world_size
-from .mixers import build_mixer, linear, _param
+from .mixers import build_mixer, linear, linear_f32, _param
 
 
 @dataclass(frozen=True)
@@ -181,7 +181,7 @@ class HybridForCausalLM(nn.Module):
         if batch.logits_indices is not None:
             x = x[batch.logits_indices]
         xn = ops.rms_norm_f32(x, self.final_norm, self.cfg.rms_norm_eps, self.dtype)
-        return linear(xn, self.head).float() * self.cfg.logit_scale
+        return linear_f32(xn, self.head) * self.cfg.logit_scale
 
     # ------------------------------------------------------------ weights
     def load_hf_state_dict(self, tensors: dict) -> None:

@@ -42,7 +42,7 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return F.linear(x, w)
 
 
-_MM_OUT_DTYPE = [True]  # torch.mm(..., out_dtype=) available
+_MM_OUT_DTYPE = {}  # device type -> torch.mm(..., out_dtype=) available
 
 
 def linear_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
@@ -50,11 +50,11 @@ def linear_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     fp32 accumulate, no rounding of the result)."""
     if x.dtype == torch.float32:
         return F.linear(x, w)
-    if _MM_OUT_DTYPE[0]:
+    if _MM_OUT_DTYPE.get(x.device.type, True):
         try:
             return torch.mm(x, w.t(), out_dtype=torch.float32)
         except (TypeError, RuntimeError):
-            _MM_OUT_DTYPE[0] = False
+            _MM_OUT_DTYPE[x.device.type] = False
     return F.linear(x, w).float()
 
 
