@@ -295,3 +295,57 @@ def test_long_portions_cross_the_recurrent_chunks(tmp_path, device, dtype):
     got = replay(eng, tmp_path, steps)
     assert rel_err(got["a"], orc.run(ta)) < TOL[dtype]
     assert rel_err(got["b"], orc.run(tb)) < TOL[dtype]
+
+
+def random_model(seed):
+    """A random layer list with sizes off the beaten path: widths that are
+    not multiples of 8 or 64, head sizes with and without a matrix-core
+    kernel, unequal q/k and value sizes, large and tiny state sizes, dt
+    ranks on both sides of the GEMM threshold, 1 to 5 conv taps."""
+    import random
+
+    r = random.Random(seed)
+    width = r.choice([40, 56, 100, 128, 192])
+    layers = []
+    for _ in range(r.randint(2, 5)):
+        mlp = r.choice([None, {"kind": "dense", "ff": r.choice([24, 72, 160])}])
+        kind = r.choice(["attention", "lightning", "mamba1"])
+        if kind == "attention":
+            kv = r.choice([1, 2, 3])
+            heads = kv * r.choice([1, 2, 4, 9])
+            dim = r.choice([8, 32, 40, 64, 96])
+            vdim = r.choice([dim, dim, 16, 48])
+            layers.append(attn(heads=heads, kv=kv, dim=dim, vdim=vdim,
+                               rot=r.choice([0, 2, dim // 2, dim]),
+                               base=r.choice([100.0, 10000.0, 1e6]),
+                               scale=r.choice([dim ** -0.5, 0.05, 0.4]), mlp=mlp))
+        elif kind == "lightning":
+            heads = r.choice([1, 2, 5])
+            dim, vdim = r.choice([(8, 8), (32, 32), (64, 64), (24, 40), (64, 128), (32, 64)])
+            layers.append(lightning(heads=heads, dim=dim, vdim=vdim,
+                                    decay=[r.choice([1.0, 0.999, 0.9, 0.3]) for _ in range(heads)],
+                                    mlp=mlp))
+        else:
+            layers.append(mamba(inner=r.choice([24, 64, 136]), state=r.choice([1, 4, 16, 48, 80]),
+                                dt_rank=r.choice([1, 4, 8, 24]), conv=r.randint(1, 5), mlp=mlp))
+    return model_cfg(layers, width=width, vocab=r.choice([64, 200]),
+                     eps=r.choice([1e-6, 1e-5, 1e-2]), logit_scale=r.choice([0.5, 1.0, 3.0]))
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("seed", range(8))
+def test_random_models(tmp_path, device, dtype, seed):
+    cfg = random_model(seed)
+    w = write_checkpoint(tmp_path / "m", cfg, seed=seed)
+    V = cfg["vocab"]
+    ta, tb = toks(150, V, seed=40 + seed), toks(70, V, seed=60 + seed)
+    orc = Oracle(cfg, w)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=256)
+    steps = [[("a", ta[:130], False)],
+             [("a", ta[130:131], False), ("b", tb[:66], False)],
+             [("a", ta[131:132], False), ("b", tb[66:67], False)],
+             [("a", ta[132:133], False)], [("a", ta[133:134], False)],
+             [("a", ta[134:], True), ("b", tb[67:], True)]]
+    got = replay(eng, tmp_path, steps)
+    assert rel_err(got["a"], orc.run(ta)) < TOL[dtype]
+    assert rel_err(got["b"], orc.run(tb)) < TOL[dtype]
