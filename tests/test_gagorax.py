@@ -352,3 +352,39 @@ def test_random_models(tmp_path, device, dtype, seed):
     tol = 2 * TOL[dtype] if dtype == "bfloat16" else TOL[dtype]
     assert rel_err(got["a"], orc.run(ta)) < tol
     assert rel_err(got["b"], orc.run(tb)) < tol
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("dim", [64, 128])
+def test_long_prompt_deep_kv(tmp_path, device, dtype, dim):
+    """A prompt long enough that the 256-row attention kernel splits its key
+    range into parts (the sink must count once) and decoding reads many
+    pages in several partitions."""
+    cfg = model_cfg([attn(heads=2, kv=1, dim=dim, vdim=dim, mlp=FF), lightning(heads=1, dim=32, vdim=32, decay=(0.99,)),
+                     mamba(inner=64, state=16, dt_rank=8, conv=4)], width=64)
+    w = write_checkpoint(tmp_path / "m", cfg, seed=dim + 1)
+    t = toks(1210, seed=8)
+    want = Oracle(cfg, w).run(t)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=1280)
+    steps = [[("a", t[:1200], False)]] + [[("a", [x], k == 9)] for k, x in enumerate(t[1200:])]
+    got = replay(eng, tmp_path, steps)["a"]
+    assert rel_err(got, want) < TOL[dtype]
+
+
+def test_preemption_recomputes_state(tmp_path):
+    """A page pool too small for all requests: sequences are preempted
+    (pages and state slot given back) and recomputed; the tokens must equal
+    those of an engine with room for everything."""
+    from arks_amd.engine import SamplingParams
+
+    write_checkpoint(tmp_path / "m", MIXED, seed=12)
+    prompts = [toks(30, seed=70 + i) for i in range(3)]
+    sp = SamplingParams(max_tokens=40, ignore_eos=True)
+    big = make_engine(tmp_path / "m", "cpu", "float32", max_tokens=512)
+    want = big.generate(prompts, sp)
+    small = make_engine(tmp_path / "m", "cpu", "float32", max_tokens=160)
+    got = small.generate(prompts, sp)
+    assert small.scheduler.num_preemptions > 0
+    assert got == want
+    assert small.runner.state_slots.num_free == 4
+    assert small.scheduler.allocator.num_free == small.runner.num_blocks
