@@ -193,9 +193,8 @@ class MoEMLP(nn.Module):
         # fused [gate|up] and down per local expert, stored PRE-TRANSPOSED
         # ([in, out] per expert) so every MoE GEMM is an NN strided bmm /
         # mm with contiguous operands: strided bmm with a transposed-VIEW B
-        # memory-faults on this ROCm stack at prefill shapes
-        # (scripts/probe_bmm_fault.py — all tb=True variants die, contiguous
-        # B passes), and NN needs no per-call transpose copies.
+        # memory-faults on this ROCm stack at prefill shapes (contiguous B
+        # passes), and NN needs no per-call transpose copies.
         self.w13 = nn.Parameter(
             torch.empty(self.local_experts, self.hidden, 2 * self.inter,
                         dtype=dtype), requires_grad=False,

@@ -311,7 +311,7 @@ def test_qwen2_moe_shared_expert_logits_match_transformers(tmp_path):
 
 def test_wide_expert_grouped_dispatch_matches_naive():
     """E=40 (>32) sparse grouped dispatch — the path that memory-faulted on
-    HW with transposed-view bmm operands (scripts/probe_bmm_fault.py) — must
+    HW with transposed-view bmm operands — must
     match a naive per-token fp32 loop."""
     import dataclasses
 
