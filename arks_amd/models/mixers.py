@@ -82,6 +82,9 @@ def rotary_inv_freq(base: float, ndims: int) -> torch.Tensor:
                      -2.0 * i / ndims).float()
 
 
+_DECODE_TILES: dict = {}
+
+
 class SinkRotaryAttention(nn.Module):
     def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
                  vdim: int, scale: float, rot_base: float, rot_dims: int,
@@ -120,12 +123,21 @@ class SinkRotaryAttention(nn.Module):
     def _tiles(self, batch: ForwardBatch, q):
         """Work lists of the MFMA kernels: host-built once per step and head
         layout (batch.tile_cache), shared by every layer of that layout.
-        None where the general kernel runs (CPU, float32, other sizes,
-        graph-captured decode steps, whose lengths are not known on the
-        host)."""
-        if (not q.is_cuda or q.dtype != torch.bfloat16 or self.D != self.V
-                or batch.kv_lens_list is None):
+        None where the general kernel runs (CPU, float32, other sizes).
+        A captured decode graph has no host lengths, but its work list is
+        static — one 64-row tile per sequence — and is kept for the life of
+        the process, since the graph holds its address."""
+        if not q.is_cuda or q.dtype != torch.bfloat16 or self.D != self.V:
             return None
+        if batch.kv_lens_list is None:
+            if batch.max_q_len != 1:
+                return None
+            B = batch.seq_lens.shape[0]
+            key = (B, self.H, self.G, self.D, q.device.index)
+            if key not in _DECODE_TILES:
+                _DECODE_TILES[key] = ops.sink_attention_tiles(
+                    [1] * B, [1] * B, self.H, self.G, self.D, q.device)
+            return _DECODE_TILES[key]
         key = (self.H, self.G, self.D)
         if key not in batch.tile_cache:
             batch.tile_cache[key] = ops.sink_attention_tiles(
