@@ -497,3 +497,36 @@ def test_cli_flags_map_to_engine_config():
     cfg2 = build_engine_config(args2)
     assert cfg2.preset == "tiny" and cfg2.model_path is None
     assert cfg2.enable_prefix_caching is True
+
+
+def test_gagorax_preset_serves_completions():
+    """A layer-list model (recurrent state slots, no prefix reuse) behind
+    the same HTTP front: a completion and a streamed chat, twice, so slots
+    and pages are taken and given back."""
+    cfg = EngineConfig(preset="tiny-gagorax", device="cpu", kv_cache_blocks=64,
+                       max_model_len=256, max_num_seqs=2)
+    engine = AsyncEngine(cfg, model_name="g")
+    mc = cfg.model_config()
+    app = create_app(engine, "g", ByteTokenizer(mc.vocab_size, mc.eos_token_id))
+
+    async def fn(client):
+        for _ in range(2):
+            r = await client.post("/v1/completions", json={
+                "model": "g", "prompt": "state", "max_tokens": 5, "temperature": 0})
+            assert r.status_code == 200, r.text
+            assert r.json()["usage"]["completion_tokens"] == 5
+            first = r.json()["choices"][0]["text"]
+        r = await client.post("/v1/completions", json={
+            "model": "g", "prompt": "state", "max_tokens": 5, "temperature": 0})
+        assert r.json()["choices"][0]["text"] == first  # reused slot, same text
+        async with client.stream("POST", "/v1/chat/completions", json={
+                "model": "g", "messages": [{"role": "user", "content": "hi"}],
+                "max_tokens": 4, "temperature": 0.8, "stream": True}) as resp:
+            assert resp.status_code == 200
+            body = "".join([chunk async for chunk in resp.aiter_text()])
+        assert "[DONE]" in body
+
+    run_with_client(app, fn)
+    sched = engine.engine.scheduler if hasattr(engine, "engine") else None
+    if sched is not None:
+        assert sched.state_slots.num_free == 2
