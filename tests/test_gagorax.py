@@ -248,7 +248,8 @@ def test_greedy_generation_through_the_scheduler(tmp_path, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("dim,heads,kv", [(32, 4, 2), (64, 8, 1), (96, 2, 2), (128, 4, 2)])
+@pytest.mark.parametrize("dim,heads,kv", [(32, 4, 2), (64, 8, 1), (96, 2, 2), (128, 4, 2),
+                                           (256, 2, 1), (64, 9, 1)])
 def test_attention_head_sizes_of_the_mfma_kernels(tmp_path, device, dtype, dim, heads, kv):
     """Equal q/k and value sizes the matrix-core kernels are built for: a
     long prompt (the 256-row kernel where it exists), short portions (the

@@ -282,7 +282,7 @@ def test_chunk_parallel_scans_equal_row_by_row(dtype, lens):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("D,V", [(32, 32), (64, 128), (128, 128)])
+@pytest.mark.parametrize("D,V", [(32, 32), (64, 64), (64, 128), (128, 64), (128, 128)])
 def test_lightning_matrix_core_prefill_equals_general_kernel(D, V):
     """bf16 rows, head sizes the matrix-core kernels are built for: chunk
     ends of 1, 63, 64 and 65 rows, decays 1, 0 and in between, old state."""
