@@ -91,6 +91,7 @@ class LLMEngine:
     def extract_prefilled(self, request_id: str):
         """After a hold_pages request finished (1 token), pull its KV pages
         for transfer and release them. Returns (prompt_len, kv tensor)."""
+        self._no_state_transfer()
         seq = self.scheduler.take_held(request_id)
         if seq is None:
             raise KeyError(f"no held sequence {request_id!r}")
@@ -115,6 +116,7 @@ class LLMEngine:
         computed remotely. Injects the pages and enters RUNNING directly."""
         from .kv_cache import BlockAllocator
 
+        self._no_state_transfer()
         seq = Sequence(prompt_token_ids, sampling, request_id, arrival_time)
         need = BlockAllocator.blocks_needed(seq.num_prompt_tokens, self.cfg.block_size)
         if not self.scheduler.allocator.can_allocate(need):
@@ -134,6 +136,13 @@ class LLMEngine:
             seq.status = SeqStatus.RUNNING
             self.scheduler.running.append(seq)
         return seq
+
+    def _no_state_transfer(self) -> None:
+        if self.runner.seq_state:
+            raise NotImplementedError(
+                "prefill/decode disaggregation moves KV pages only; "
+                f"{self.model_cfg.architecture} also keeps per-sequence "
+                "recurrent state")
 
     def has_work(self) -> bool:
         return self.scheduler.has_work()
