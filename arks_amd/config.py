@@ -151,8 +151,9 @@ class ModelConfig:
 @dataclass
 class HybridModelConfig:
     """Layer-list decoders: config.json names one architecture and lists the
-    layers, each with its mixer type ("attention", "lightning", "mamba1"),
-    the mixer's sizes and an optional feed-forward. Every size and every
+    layers, each with its mixer type ("attention", "lightning", "mamba1",
+    "parallel"), the mixer's sizes and an optional feed-forward (dense, or
+    "moe" where the architecture has one). Every size and every
     per-model constant comes from that file; what the architecture itself
     fixes (block arrangement, activation, rotary pairing) lives with the
     model code (arks_amd/models/hybrid.py)."""
@@ -166,12 +167,22 @@ class HybridModelConfig:
     eos_token_id: int = -1  # the format defines no end token
     bos_token_id: int = -1
     torch_dtype: str = "bfloat16"
+    # stream arrangement (Fusolix): copies of the residual, taps of the
+    # input convolution (0 = none), factor on the embedding rows
+    streams: int = 1
+    conv_taps: int = 0
+    embed_scale: float = 1.0
 
     # what the engine asks of any model config
-    num_local_experts = 0
     sliding_window = None
 
-    ARCHITECTURES = ("Gagorax",)
+    ARCHITECTURES = ("Gagorax", "Fusolix")
+    MOE_ARCHITECTURES = ("Fusolix",)
+
+    @property
+    def num_local_experts(self) -> int:
+        return max([l["mlp"]["router"]["experts"] for l in self.layers or []
+                    if l.get("mlp") and l["mlp"].get("kind") == "moe"] or [0])
 
     @classmethod
     def matches(cls, cfg: dict) -> bool:
@@ -182,8 +193,10 @@ class HybridModelConfig:
         layers = []
         for entry in cfg["layers"]:
             mlp = entry.get("mlp")
-            if mlp is not None and mlp.get("kind", "dense") != "dense":
-                raise ValueError(f"unknown feed-forward kind {mlp.get('kind')!r}")
+            kind = mlp.get("kind", "dense") if mlp is not None else "dense"
+            if kind != "dense" and not (
+                    kind == "moe" and cfg["architecture"] in cls.MOE_ARCHITECTURES):
+                raise ValueError(f"unknown feed-forward kind {kind!r}")
             layers.append({"type": entry["type"], "mixer": dict(entry["mixer"]),
                            "mlp": dict(mlp) if mlp is not None else None})
         return cls(
@@ -195,13 +208,21 @@ class HybridModelConfig:
             logit_scale=float(cfg.get("logit_scale", 1.0)),
             eos_token_id=int(cfg.get("eos_token_id", -1)),
             bos_token_id=int(cfg.get("bos_token_id", -1)),
+            streams=int(cfg.get("streams", 1)),
+            conv_taps=int((cfg.get("canon") or {}).get("taps", 0)),
+            embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
         )
 
     def to_dict(self) -> dict:
-        return {"architecture": self.architecture, "vocab": self.vocab_size,
-                "width": self.hidden_size, "layers": self.layers,
-                "norm": {"eps": self.rms_norm_eps},
-                "logit_scale": self.logit_scale}
+        out = {"architecture": self.architecture, "vocab": self.vocab_size,
+               "width": self.hidden_size, "layers": self.layers,
+               "norm": {"eps": self.rms_norm_eps},
+               "logit_scale": self.logit_scale}
+        if self.architecture == "Fusolix":
+            out.update({"streams": self.streams,
+                        "canon": {"taps": self.conv_taps},
+                        "embedding": {"scale": self.embed_scale}})
+        return out
 
     @property
     def num_hidden_layers(self) -> int:

@@ -21,6 +21,10 @@ _REGISTRY = {
     # layer-list decoder: attention / lightning / mamba1 mixers, fp32
     # residual, token shift + gated residual (models/hybrid.py)
     "Gagorax": HybridForCausalLM,
+    # layer-list decoder: residual in weighted copies, layer norm + short
+    # input convolution, window/pooled attention beside retention, clamped
+    # GLU or group-routed experts (models/hybrid.py StreamBlock)
+    "Fusolix": HybridForCausalLM,
 }
 
 

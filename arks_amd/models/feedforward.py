@@ -1,0 +1,111 @@
+"""Feed-forward sublayers of the layer-list decoders, each with its
+constants as constructor parameters:
+
+- ClampedGLU: W_down act(W_gate x, W_up x) with the gate capped from above,
+  the up branch clamped on both sides and offset by one:
+  g = min(gate, limit), u = clamp(up, -limit, limit),
+  act = g * sigmoid(alpha g) * (u + 1). Gate and up are one fused GEMM.
+- GroupedMoE: `experts` small silu-GLU feed-forwards of which every row
+  uses `top`; the router's softmax runs over all experts in fp32, experts
+  form `groups` runs of neighbours and only those of the `keep` groups with
+  the best single score can be chosen; the chosen scores are renormalised.
+  Expert weights are kept pre-transposed ([in, out] per expert) like the
+  framework's other sparse feed-forward (models/llama_family.py MoEMLP), and
+  the two execution paths are the same: below DENSE_TOKENS rows every expert
+  runs on every row as two batched GEMMs (data-independent shapes, so the
+  step can be captured), above it rows are sorted by expert and run as a
+  capacity-padded batched GEMM.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from .. import ops
+from .mixers import _param, linear, linear_f32
+
+
+class ClampedGLU(nn.Module):
+    def __init__(self, width: int, ff: int, limit: float, dtype,
+                 alpha: float = 1.702):
+        super().__init__()
+        self.ff, self.limit, self.alpha = ff, float(limit), float(alpha)
+        self.gate_up = _param(2 * ff, width, dtype=dtype)
+        self.down = _param(width, ff, dtype=dtype)
+
+    def weight_map(self) -> dict:
+        return {"gate": (self.gate_up, 0), "up": (self.gate_up, self.ff),
+                "down": (self.down, 0)}
+
+    def forward(self, h, batch=None, cache=None) -> torch.Tensor:
+        gu = linear(h, self.gate_up)
+        return linear(ops.glu_act(gu, "clamped", self.limit, self.alpha),
+                      self.down)
+
+
+class GroupedMoE(nn.Module):
+    DENSE_TOKENS = 256  # see models/llama_family.py MoEMLP.DENSE_TOKENS
+
+    def __init__(self, width: int, experts: int, ff: int, top: int,
+                 groups: int, keep: int, dtype):
+        super().__init__()
+        assert experts % groups == 0 and keep <= groups
+        assert top <= keep * (experts // groups)
+        self.E, self.ff, self.top = experts, ff, top
+        self.groups, self.keep, self.width = groups, keep, width
+        self.router = _param(experts, width, dtype=dtype)
+        self.w13 = _param(experts, width, 2 * ff, dtype=dtype)
+        self.w2 = _param(experts, ff, width, dtype=dtype)
+
+    def weight_map(self) -> dict:
+        m = {"router": (self.router, 0)}
+        W, ff = self.width, self.ff
+        for e in range(self.E):
+            # (param, row, col, shape, expert index, transposed)
+            m[f"e{e}.gate"] = (self.w13, 0, 0, (ff, W), e, True)
+            m[f"e{e}.up"] = (self.w13, ff, 0, (ff, W), e, True)
+            m[f"e{e}.down"] = (self.w2, 0, 0, (W, ff), e, True)
+        return m
+
+    def forward(self, h, batch=None, cache=None) -> torch.Tensor:
+        T = h.shape[0]
+        E, ff, W, k = self.E, self.ff, self.width, self.top
+        z = linear_f32(h, self.router)  # fp32 logits
+        weights, ids = ops.moe_route_grouped(z, k, self.groups, self.keep)
+        if T <= self.DENSE_TOKENS:
+            xb = h.unsqueeze(0).expand(E, T, W)
+            gu = torch.bmm(xb, self.w13)
+            a = ops.glu_act(gu.view(E * T, 2 * ff), "swiglu")
+            y = torch.bmm(a.view(E, T, ff), self.w2)
+            return ops.moe_mix_seq(y, weights, ids)
+        # rows sorted by expert, every expert's segment padded to the
+        # heaviest one's length (one host read of the segment table)
+        flat = ids.reshape(-1).long()
+        order = torch.argsort(flat, stable=True)
+        tok = torch.div(order, k, rounding_mode="floor")
+        counts = torch.bincount(flat, minlength=E)
+        starts = torch.cumsum(counts, 0) - counts
+        cap = int(counts.max())
+        ar = torch.arange(cap, device=h.device)[None, :]
+        src = torch.where(ar < counts[:, None], starts[:, None] + ar,
+                          torch.zeros_like(ar)).reshape(-1)
+        xp = h[tok[src]].view(E, cap, W)
+        gu = torch.bmm(xp, self.w13)
+        a = ops.glu_act(gu.view(E * cap, 2 * ff), "swiglu")
+        y = torch.bmm(a.view(E, cap, ff), self.w2).view(E * cap, W)
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(T * k, device=h.device)
+        rows = flat * cap + (inv - starts[flat])
+        return ops.moe_mix_rows_seq(y, weights, rows.view(T, k).to(torch.int32))
+
+
+def build_feedforward(mlp: dict, width: int, dtype) -> nn.Module:
+    kind = mlp.get("kind", "dense")
+    if kind == "dense":
+        return ClampedGLU(width, mlp["ff"], mlp["limit"], dtype)
+    if kind == "moe":
+        r = mlp["router"]
+        return GroupedMoE(width, r["experts"], mlp["expert"]["ff"], r["top"],
+                          r["groups"]["count"], r["groups"]["keep"], dtype)
+    raise ValueError(f"unknown feed-forward kind {kind!r}")

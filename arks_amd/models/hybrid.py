@@ -2,7 +2,22 @@
 with one mixer of arks_amd/models/mixers.py and an optional dense
 feed-forward, around an fp32 residual stream.
 
-What an architecture fixes is a BlockArrangement; Gagorax's is:
+What an architecture fixes is a BlockArrangement. Fusolix's is:
+  - the residual is `streams` weighted copies xs[s] (all equal to the scaled
+    embedding at first); sublayer q of a layer reads u = sum_s in_q[s] xs[s],
+    and its result y rewrites every copy from all old ones:
+    xs[t] <- sum_s mix_q[s, t] xs[s] + out_q[t] y; the model's output is
+    the sum of the copies
+  - layer norm (weight and bias) on each sublayer's INPUT, then a short
+    causal depthwise convolution added to its own input (h + conv(h)); its
+    last taps-1 inputs are per-sequence state, per layer and sublayer
+  - mixer "parallel" (models/mixers.py ParallelMixer), feed-forward
+    ClampedGLU or GroupedMoE (models/feedforward.py)
+  Kernel plan per sublayer: stream_mix_norm (applies the previous
+  sublayer's y to the copies, reads the next input and normalises it, one
+  pass) -> short_conv_residual -> sublayer.
+
+Gagorax's is:
   - the sublayers read the residual x itself and the RMS norm sits on each
     sublayer's OUTPUT:  x += norm(sublayer(x)) * w
   - token shift: the mixer reads x_t + (x_{t-1} - x_t) * s (x_{-1} = 0);
@@ -36,6 +51,7 @@ from .. import ops
 from ..config import HybridModelConfig
 from ..engine.forward_batch import ForwardBatch
 from ..parallel.comm import get_tp_world_size
+from .feedforward import build_feedforward
 from .mixers import build_mixer, linear, linear_f32, _param
 
 
@@ -43,10 +59,17 @@ from .mixers import build_mixer, linear, linear_f32, _param
 class BlockArrangement:
     token_shift: bool = True
     gated_residual: bool = True
-    norm_place: str = "output"  # only sublayer-output norms so far
+    # "output": RMS norm on each sublayer's result (HybridBlock);
+    # "input": layer norm with bias in front of each sublayer, residual in
+    # weighted copies, short input convolution (StreamBlock)
+    norm_place: str = "output"
 
 
-ARRANGEMENTS = {"Gagorax": BlockArrangement()}
+ARRANGEMENTS = {
+    "Gagorax": BlockArrangement(),
+    "Fusolix": BlockArrangement(token_shift=False, gated_residual=False,
+                                norm_place="input"),
+}
 
 
 class HybridBlock(nn.Module):
@@ -113,6 +136,58 @@ class HybridBlock(nn.Module):
             ops.gated_norm_residual(x, y, g, self.rg2_b, self.norm2, self.eps, None)
 
 
+class StreamBlock(nn.Module):
+    """One layer of the stream arrangement: up to two sublayers (mixer,
+    feed-forward), each with its layer norm, input convolution and the
+    three small tensors that connect it to the residual copies."""
+
+    def __init__(self, width: int, spec: dict, streams: int, taps: int,
+                 eps: float, dtype):
+        super().__init__()
+        f32 = torch.float32
+        self.width, self.taps, self.eps = width, taps, eps
+        self.mixer = build_mixer(spec["type"], spec["mixer"], width, eps, dtype)
+        self.ffn = (build_feedforward(spec["mlp"], width, dtype)
+                    if spec.get("mlp") is not None else None)
+        self.nsub = 2 if self.ffn is not None else 1
+        for q in range(1, self.nsub + 1):
+            setattr(self, f"norm{q}", _param(width, dtype=f32))
+            setattr(self, f"norm{q}_b", _param(width, dtype=f32))
+            setattr(self, f"hc{q}_in", _param(streams, dtype=f32))
+            setattr(self, f"hc{q}_out", _param(streams, dtype=f32))
+            setattr(self, f"hc{q}_mix", _param(streams, streams, dtype=f32))
+            if taps:
+                setattr(self, f"canon{q}", _param(width, taps, dtype=f32))
+
+    def weight_map(self) -> dict:
+        m = {"mix." + k: v for k, v in self.mixer.weight_map().items()}
+        if self.ffn is not None:
+            m.update({"mlp." + k: v for k, v in self.ffn.weight_map().items()})
+        for q in range(1, self.nsub + 1):
+            m[f"norm{q}"] = (getattr(self, f"norm{q}"), 0)
+            m[f"norm{q}.b"] = (getattr(self, f"norm{q}_b"), 0)
+            for leaf in ("in", "out", "mix"):
+                m[f"hc{q}.{leaf}"] = (getattr(self, f"hc{q}_{leaf}"), 0)
+            if self.taps:
+                m[f"canon{q}"] = (getattr(self, f"canon{q}"), 0)
+        return m
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        out = {"mix." + k: v
+               for k, v in self.mixer.cache_layout(block_size, dtype).items()}
+        if self.taps > 1:
+            for q in range(1, self.nsub + 1):
+                out[f"canon{q}"] = ("slot", (self.taps - 1, self.width),
+                                    torch.float32)
+        return out
+
+    def sublayers(self):
+        """(index, module, cache prefix) of each sublayer in order."""
+        yield 1, self.mixer, "mix."
+        if self.ffn is not None:
+            yield 2, self.ffn, None
+
+
 class HybridForCausalLM(nn.Module):
     supports_float32 = True
     has_sequence_state = True  # engine: state slots, no prefix reuse
@@ -125,14 +200,26 @@ class HybridForCausalLM(nn.Module):
         self.cfg, self.dtype = cfg, dtype
         arr = ARRANGEMENTS[cfg.architecture]
         W = cfg.hidden_size
+        self.arr = arr
         self.embed = _param(cfg.vocab_size, W, dtype=dtype)
-        self.layers = nn.ModuleList(
-            HybridBlock(W, spec, cfg.rms_norm_eps, dtype, arr)
-            for spec in cfg.layers)
+        if arr.norm_place == "input":
+            self.layers = nn.ModuleList(
+                StreamBlock(W, spec, cfg.streams, cfg.conv_taps,
+                            cfg.rms_norm_eps, dtype)
+                for spec in cfg.layers)
+        else:
+            self.layers = nn.ModuleList(
+                HybridBlock(W, spec, cfg.rms_norm_eps, dtype, arr)
+                for spec in cfg.layers)
         self.final_norm = _param(W, dtype=torch.float32)
         self.head = _param(cfg.vocab_size, W, dtype=dtype)
         self._wmap = {"embed": (self.embed, 0), "head": (self.head, 0),
                       "final.norm": (self.final_norm, 0)}
+        if arr.norm_place == "input":
+            self.final_norm_b = _param(W, dtype=torch.float32)
+            self._wmap["final.norm.b"] = (self.final_norm_b, 0)
+            self.register_buffer("sum_w", torch.ones(cfg.streams),
+                                 persistent=False)
         for i, layer in enumerate(self.layers):
             for k, v in layer.weight_map().items():
                 self._wmap[f"l{i}.{k}"] = v
@@ -173,6 +260,8 @@ class HybridForCausalLM(nn.Module):
     # ------------------------------------------------------------ forward
     def forward(self, batch: ForwardBatch, caches: list) -> torch.Tensor:
         """fp32 logits for batch.logits_indices rows (all rows if None)."""
+        if self.arr.norm_place == "input":
+            return self._forward_streams(batch, caches)
         x = self.embed[batch.input_ids].float()
         for i, layer in enumerate(self.layers):
             layer(x, batch, caches[i], self.dtype)
@@ -183,15 +272,70 @@ class HybridForCausalLM(nn.Module):
         xn = ops.rms_norm_f32(x, self.final_norm, self.cfg.rms_norm_eps, self.dtype)
         return linear_f32(xn, self.head) * self.cfg.logit_scale
 
+    def _forward_streams(self, batch: ForwardBatch, caches: list) -> torch.Tensor:
+        """Stream arrangement: the previous sublayer's result is applied to
+        the residual copies by the kernel that reads the next sublayer's
+        input, so each sublayer costs one pass over the copies."""
+        cfg, dtype = self.cfg, self.dtype
+        x0 = self.embed[batch.input_ids].float() * cfg.embed_scale
+        xs = x0.unsqueeze(0).repeat(cfg.streams, 1, 1)
+        pend = (None, None, None, None)  # y, its fp32 bias, mix, out
+        for i, layer in enumerate(self.layers):
+            cache = caches[i]
+            for q, module, prefix in layer.sublayers():
+                n = ops.stream_mix_norm(
+                    xs, *pend, getattr(layer, f"hc{q}_in"),
+                    getattr(layer, f"norm{q}"), getattr(layer, f"norm{q}_b"),
+                    layer.eps)
+                if layer.taps:
+                    h = ops.short_conv_residual(
+                        n, getattr(layer, f"canon{q}"), cache.get(f"canon{q}"),
+                        batch.cu_seqlens, batch.seq_lens, batch.state_slots,
+                        batch.token_seq, dtype)
+                else:
+                    h = n.to(dtype)
+                sub = ({k[len(prefix):]: v for k, v in cache.items()
+                        if k.startswith(prefix)} if prefix else None)
+                y = module(h, batch, sub)
+                pend = (y, getattr(module, "out_bias", None),
+                        getattr(layer, f"hc{q}_mix"),
+                        getattr(layer, f"hc{q}_out"))
+            if self.residual_tap is not None:
+                ops.stream_mix_norm(xs, *pend, None, None, None, layer.eps)
+                pend = (None, None, None, None)
+                self.residual_tap(i, xs.sum(0))
+        n = ops.stream_mix_norm(xs, *pend, self.sum_w, self.final_norm,
+                                self.final_norm_b, cfg.rms_norm_eps)
+        if batch.logits_indices is not None:
+            n = n[batch.logits_indices]
+        return linear_f32(n.to(dtype), self.head) * cfg.logit_scale
+
     # ------------------------------------------------------------ weights
+    @staticmethod
+    def _span(entry, w):
+        """The part of a parameter one checkpoint tensor fills. Entries are
+        (param, row) for row spans of fused parameters, or (param, row, col,
+        shape[, index[, transposed]]) for column spans and for slices of
+        stacked, pre-transposed parameters."""
+        p, row = entry[0], entry[1]
+        if len(entry) == 2:
+            return p.data[row:row + w.shape[0]] if w.dim() else p.data
+        col, shape = entry[2], entry[3]
+        d = p.data
+        if len(entry) > 4 and entry[4] is not None:
+            d = d[entry[4]]
+        if len(entry) > 5 and entry[5]:
+            d = d.t()
+        return d[row:row + shape[0], col:col + shape[1]]
+
     def load_hf_state_dict(self, tensors: dict) -> None:
         """Tensors by their checkpoint names ('embed', 'l<i>.mix.q', ...);
         fused parameters are filled span by span, in any order."""
         for name, w in tensors.items():
             if name not in self._wmap:
                 raise KeyError(f"unexpected tensor {name!r}")
-            p, row = self._wmap[name]
-            span = p.data[row:row + w.shape[0]] if w.dim() else p.data
+            p = self._wmap[name][0]
+            span = self._span(self._wmap[name], w)
             if span.shape != w.shape:
                 raise ValueError(f"{name}: shape {tuple(w.shape)} does not fit "
                                  f"{tuple(span.shape)}")
@@ -214,15 +358,21 @@ class HybridForCausalLM(nn.Module):
         block (benchmarks and tests; checkpoints load by name instead)."""
         dev = self.embed.device
         self._loaded.clear()
-        for name, (p, row) in self._wmap.items():
+        streams = getattr(self.cfg, "streams", 1)
+        for name, entry in self._wmap.items():
+            p, row = entry[0], entry[1]
             s = (seed * 1000003 + zlib.crc32(name.encode())) % (2 ** 63 - 1)
             g = torch.Generator(device=dev).manual_seed(s)
             leaf = name.split(".", 1)[1] if name.startswith("l") and "." in name else name
             # rows of this tensor inside its (possibly fused) parameter
-            shape = list(p.shape)
-            if p.dim() == 2:
-                nxt = sorted(r for q, r in self._wmap.values() if q is p and r > row)
-                shape[0] = (nxt[0] if nxt else p.shape[0]) - row
+            if len(entry) > 2:
+                shape = list(entry[3])
+            else:
+                shape = list(p.shape)
+                if p.dim() >= 1:
+                    nxt = sorted(e[1] for e in self._wmap.values()
+                                 if e[0] is p and len(e) == 2 and e[1] > row)
+                    shape[0] = (nxt[0] if nxt else p.shape[0]) - row
 
             def rn(std):
                 return torch.randn(shape, generator=g, device=dev,
@@ -230,6 +380,16 @@ class HybridForCausalLM(nn.Module):
 
             if leaf.endswith("norm") or leaf in ("norm1", "norm2"):
                 w = 1.0 + rn(0.1)
+            elif leaf.startswith("canon"):
+                w = rn(0.3)
+            elif leaf.startswith("hc") and leaf.endswith(".in"):
+                w = 1.0 / streams + rn(0.2)
+            elif leaf.startswith("hc") and leaf.endswith(".out"):
+                w = 1.0 + rn(0.3)
+            elif leaf.startswith("hc") and leaf.endswith(".mix"):
+                w = torch.eye(streams, device=dev) + rn(0.15)
+            elif leaf.endswith("router"):
+                w = rn(2.0 * shape[-1] ** -0.5)
             elif leaf == "shift":
                 w = torch.rand(shape, generator=g, device=dev)
             elif leaf == "mix.A_log":
@@ -239,7 +399,7 @@ class HybridForCausalLM(nn.Module):
             elif leaf.endswith(".b") or leaf == "mix.D":
                 w = rn(0.3)
             elif leaf == "embed":
-                w = rn(1.0)
+                w = rn(1.0 / getattr(self.cfg, "embed_scale", 1.0))
             else:
                 w = rn(shape[-1] ** -0.5)
             self.load_hf_state_dict({name: w})

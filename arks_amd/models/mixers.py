@@ -10,6 +10,21 @@ constructor parameters so that more than one design can use it:
   [dim x vdim] fp32 state per head and sequence, gated RMS-normed output.
 - Mamba1Mixer: short causal depthwise convolution + selective scan with an
   [inner x state] fp32 state per sequence.
+- WindowPoolAttention: grouped-query softmax attention without positions in
+  the scores, over a sliding window of recent keys plus one pooled (mean)
+  key/value per block of older positions; biases on every projection.
+- RetentionMixer: the lightning recurrence on plain rows (nothing
+  activated) with partial rotary on q and k, scaled keys, a per-head unit
+  RMS of the output and a silu gate.
+- ParallelMixer: two of the above side by side on the same input, as ONE
+  in-projection GEMM and ONE out-projection GEMM over the concatenated
+  (pre-scaled) head outputs.
+
+The last three are "split" mixers: they name the rows of their
+in-projection (in_spans) and the columns of their out-projection
+(out_cols) and do everything between in core(), so that a parent can fuse
+the projections of several of them; alone, SplitMixer.forward runs the
+same three steps with projections of their own.
 
 Every mixer maps the (already token-shifted) rows [T, width] of one engine
 step to [T, width]; rows of several sequences are packed, prompt portions
@@ -34,12 +49,12 @@ from .. import ops
 from ..engine.forward_batch import ForwardBatch
 
 
-def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """x @ w^T as a library GEMM (the decode-shaped bf16 cases go to the
-    split-K kernel when the main extension is built)."""
+def linear(x: torch.Tensor, w: torch.Tensor, b=None) -> torch.Tensor:
+    """x @ w^T (+ b) as a library GEMM (the decode-shaped bf16 cases go to
+    the split-K kernel when the main extension is built)."""
     if x.dtype == torch.bfloat16:
-        return ops.linear_bf16(x, w)
-    return F.linear(x, w)
+        return ops.linear_bf16(x, w, b)
+    return F.linear(x, w, b)
 
 
 _MM_OUT_DTYPE = {}  # device type -> torch.mm(..., out_dtype=) available
@@ -261,6 +276,215 @@ class Mamba1Mixer(nn.Module):
         return linear(y, self.o)
 
 
+class SplitMixer(nn.Module):
+    """A mixer in three parts: rows of an in-projection (in_spans: name,
+    rows, has_bias), core() from those rows to the columns of an
+    out-projection (out_cols, out_bias). With own_projections the module
+    holds both projections itself; without, a parent (ParallelMixer) holds
+    fused ones and calls core() on its slice."""
+
+    out_has_bias = False
+
+    def in_spans(self) -> list:
+        raise NotImplementedError
+
+    def _make_projections(self, width: int, dtype) -> None:
+        spans = self.in_spans()
+        rows = sum(n for _, n, _ in spans)
+        self.w_in = _param(rows, width, dtype=dtype)
+        self.b_in = (_param(rows, dtype=dtype)
+                     if any(b for _, _, b in spans) else None)
+        self.w_out = _param(width, self.out_cols, dtype=dtype)
+        self.b_out = _param(width, dtype=dtype) if self.out_has_bias else None
+
+    def weight_map(self) -> dict:
+        m, row = {}, 0
+        for name, n, has_b in self.in_spans():
+            m[name] = (self.w_in, row)
+            if has_b:
+                m[name + ".b"] = (self.b_in, row)
+            row += n
+        m["o"] = (self.w_out, 0)
+        if self.b_out is not None:
+            m["o.b"] = (self.b_out, 0)
+        return m
+
+    def forward(self, xs, batch: ForwardBatch, cache: dict) -> torch.Tensor:
+        p = linear(xs, self.w_in, self.b_in)
+        out = torch.empty((xs.shape[0], self.out_cols), dtype=xs.dtype,
+                          device=xs.device)
+        self.core(p, batch, cache, out, 1.0)
+        return linear(out, self.w_out, self.b_out)
+
+
+class WindowPoolAttention(SplitMixer):
+    """Softmax attention, query head h on key/value head h // (H/G), no
+    positions in the scores: the row at position i sees keys j with
+    0 <= i - j < window and one pooled key/value (the mean over the block,
+    taken from what the pages hold) for every block of `pool` positions
+    that ends at or before i - window. Paged k/v plus paged pooled kp/vp
+    (ops.kv_write_pooled)."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, scale: float, window: int, pool: int, dtype,
+                 bias: bool = True, own_projections: bool = True):
+        super().__init__()
+        assert heads % kv_heads == 0 and window >= 1 and pool >= 1
+        self.H, self.G, self.D, self.V = heads, kv_heads, dim, vdim
+        self.scale, self.window, self.pool = float(scale), int(window), int(pool)
+        self.bias = self.out_has_bias = bias
+        self.out_cols = heads * vdim
+        if own_projections:
+            self._make_projections(width, dtype)
+
+    def in_spans(self) -> list:
+        return [("q", self.H * self.D, self.bias),
+                ("k", self.G * self.D, self.bias),
+                ("v", self.G * self.V, self.bias)]
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        spp = ops.pool_slots_per_page(block_size, self.pool)
+        return {"k": ("paged", (self.G, block_size, self.D), dtype),
+                "v": ("paged", (self.G, block_size, self.V), dtype),
+                "kp": ("paged", (self.G, spp, self.D), dtype),
+                "vp": ("paged", (self.G, spp, self.V), dtype)}
+
+    def core(self, p, batch: ForwardBatch, cache: dict, out, out_scale) -> None:
+        H, G, D, V = self.H, self.G, self.D, self.V
+        q = p[:, :H * D].unflatten(-1, (H, D))
+        k = p[:, H * D:(H + G) * D].unflatten(-1, (G, D))
+        v = p[:, (H + G) * D:(H + G) * D + G * V].unflatten(-1, (G, V))
+        ops.kv_write_pooled(k, v, cache["k"], cache["v"], cache["kp"],
+                            cache["vp"], batch.slot_mapping, batch.positions,
+                            batch.block_tables, batch.token_seq, self.pool)
+        ops.attention_window_pool(
+            q, cache["k"], cache["v"], cache["kp"], cache["vp"],
+            batch.block_tables, batch.seq_lens, batch.cu_seqlens,
+            batch.token_seq, self.scale, self.window, self.pool,
+            out.unflatten(-1, (H, V)), out_scale, batch.max_q_len)
+
+
+class RetentionMixer(SplitMixer):
+    """S <- decay_h S + k v^T, o = S^T q per head on plain projections: q
+    and k turned by their position over their first rot_dims dims
+    (half-split pairs unless interleaved), k times k_scale after that; each
+    head's o divided by its root mean square, times silu(gate). fp32 state
+    [H, D, V] per sequence; runs the lightning kernels."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay,
+                 rot_base: float, rot_dims: int, eps: float, dtype,
+                 k_scale: float | None = None, interleaved: bool = False,
+                 own_projections: bool = True):
+        super().__init__()
+        assert len(decay) == heads and rot_dims % 2 == 0 and rot_dims <= dim
+        self.H, self.D, self.V, self.eps = heads, dim, vdim, eps
+        self.k_scale = float(dim ** -0.5 if k_scale is None else k_scale)
+        self.interleaved = interleaved
+        self.out_cols = heads * vdim
+        self.register_buffer("decay", torch.tensor(
+            [float(d) for d in decay], dtype=torch.float64).float(),
+            persistent=False)
+        self.register_buffer(
+            "inv_freq", rotary_inv_freq(rot_base, rot_dims) if rot_dims else None,
+            persistent=False)
+        if own_projections:
+            self._make_projections(width, dtype)
+
+    def in_spans(self) -> list:
+        HD, HV = self.H * self.D, self.H * self.V
+        return [("q", HD, False), ("k", HD, False), ("v", HV, False),
+                ("g", HV, False)]
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        return {"S": ("slot", (self.H, self.D, self.V), torch.float32)}
+
+    def core(self, p, batch: ForwardBatch, cache: dict, out, out_scale) -> None:
+        T = p.shape[0]
+        H, D, V = self.H, self.D, self.V
+        q = p[:, :H * D].unflatten(-1, (H, D))
+        k = p[:, H * D:2 * H * D].unflatten(-1, (H, D))
+        v = p[:, 2 * H * D:2 * H * D + H * V].unflatten(-1, (H, V))
+        g = p[:, 2 * H * D + H * V:2 * H * D + 2 * H * V]
+        o = ops.retention_scan(
+            q, k, v, self.decay, cache["S"], batch.cu_seqlens, batch.seq_lens,
+            batch.state_slots, batch.positions, self.inv_freq,
+            self.interleaved, self.k_scale, batch.max_q_len,
+            step_chunks(batch, p.device))
+        ops.head_norm_gate(o.view(T, H * V), g, self.eps, H, out, out_scale)
+
+
+class ParallelMixer(nn.Module):
+    """left_scale * left(h) + right_scale * right(h) for two split mixers:
+    one GEMM projects h for both, each core() writes its head outputs,
+    already multiplied by its scale, into its columns of one buffer, and
+    one GEMM over [W_o,left | W_o,right] sums the two results. The left
+    out-projection's bias (times its scale) is handed to the caller as
+    out_bias (fp32), to be added where the result meets the residual."""
+
+    def __init__(self, width: int, left: SplitMixer, right: SplitMixer,
+                 left_scale: float, right_scale: float, dtype):
+        super().__init__()
+        self.left, self.right = left, right
+        self.scales = (float(left_scale), float(right_scale))
+        self._spans = [("left." + n, r, b) for n, r, b in left.in_spans()] + \
+                      [("right." + n, r, b) for n, r, b in right.in_spans()]
+        self.rows = (sum(r for _, r, _ in left.in_spans()),
+                     sum(r for _, r, _ in right.in_spans()))
+        self.cols = (left.out_cols, right.out_cols)
+        self.w_in = _param(sum(self.rows), width, dtype=dtype)
+        self.b_in = (_param(sum(self.rows), dtype=dtype)
+                     if any(b for _, _, b in self._spans) else None)
+        self.w_out = _param(width, sum(self.cols), dtype=dtype)
+        self.o_b = {side: _param(width, dtype=torch.float32)
+                    for side, m in (("left", left), ("right", right))
+                    if m.out_has_bias}
+        for side, p in self.o_b.items():
+            self.register_parameter("o_b_" + side, p)
+        self.out_bias = (_param(width, dtype=torch.float32)
+                         if self.o_b else None)
+
+    def weight_map(self) -> dict:
+        m, row = {}, 0
+        for name, n, has_b in self._spans:
+            m[name] = (self.w_in, row)
+            if has_b:
+                m[name + ".b"] = (self.b_in, row)
+            row += n
+        width = self.w_out.shape[0]
+        m["left.o"] = (self.w_out, 0, 0, (width, self.cols[0]))
+        m["right.o"] = (self.w_out, 0, self.cols[0], (width, self.cols[1]))
+        for side in self.o_b:
+            m[side + ".o.b"] = (getattr(self, "o_b_" + side), 0)
+        return m
+
+    def finish_loading(self) -> None:
+        if self.out_bias is not None:
+            total = torch.zeros_like(self.out_bias.data)
+            for side, scale in zip(("left", "right"), self.scales):
+                if side in self.o_b:
+                    total += scale * getattr(self, "o_b_" + side).data
+            self.out_bias.data.copy_(total)
+
+    def cache_layout(self, block_size: int, dtype) -> dict:
+        out = {"left." + k: v
+               for k, v in self.left.cache_layout(block_size, dtype).items()}
+        out.update({"right." + k: v for k, v in
+                    self.right.cache_layout(block_size, dtype).items()})
+        return out
+
+    def forward(self, xs, batch: ForwardBatch, cache: dict) -> torch.Tensor:
+        p = linear(xs, self.w_in, self.b_in)
+        out = torch.empty((xs.shape[0], sum(self.cols)), dtype=xs.dtype,
+                          device=xs.device)
+        lc = {k[5:]: v for k, v in cache.items() if k.startswith("left.")}
+        rc = {k[6:]: v for k, v in cache.items() if k.startswith("right.")}
+        self.left.core(p[:, :self.rows[0]], batch, lc, out[:, :self.cols[0]],
+                       self.scales[0])
+        self.right.core(p[:, self.rows[0]:], batch, rc, out[:, self.cols[0]:],
+                        self.scales[1])
+        return linear(out, self.w_out)
+
+
 def build_mixer(kind: str, m: dict, width: int, eps: float, dtype) -> nn.Module:
     if kind == "attention":
         return SinkRotaryAttention(
@@ -272,4 +496,16 @@ def build_mixer(kind: str, m: dict, width: int, eps: float, dtype) -> nn.Module:
     if kind == "mamba1":
         return Mamba1Mixer(width, m["inner"], m["state"], m["dt_rank"],
                            m["conv"], dtype)
+    if kind == "parallel":
+        L, R = m["left"], m["right"]
+        left = WindowPoolAttention(
+            width, L["heads"], L["kv_heads"], L["dim"], L["vdim"], L["scale"],
+            L["mask"]["size"], L["mask"]["pool"], dtype,
+            own_projections=False)
+        right = RetentionMixer(
+            width, R["heads"], R["dim"], R["vdim"], R["decay"],
+            R["rot"]["base"], R["rot"]["dims"], eps, dtype,
+            own_projections=False)
+        return ParallelMixer(width, left, right, m["left_scale"],
+                             m["right_scale"], dtype)
     raise ValueError(f"unknown mixer type {kind!r}")

@@ -735,6 +735,11 @@ def scan_chunks(q_lens: list[int], device, chunk: int = SCAN_CHUNK) -> dict:
             "slots": t(list(range(len(rows)))), "off": t(off)}
 
 
+# the lightning kernels' input convention without positions: rows pass
+# through silu (no positions, no rotary table, pairing, key scale)
+_SILU_ROWS = (None, None, False, 1.0)
+
+
 def lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
                    max_q_len=0, chunks=None):
     """chunks (scan_chunks of this step): run the prefill chunk-parallel."""
@@ -750,21 +755,25 @@ def lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
             # bf16 rows with head sizes the matrix-core kernels are built
             # for run those; the general kernel does the same two passes
             mfma = (q.dtype == torch.bfloat16 and use_lightning_mfma
-                    and S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 1))
+                    and S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 1,
+                                         *_SILU_ROWS))
             if not mfma:
                 S.lightning_scan(out, q, k, v, decay, part, c["cu"],
-                                 c["lens0"], c["slots"], SCAN_CHUNK)
+                                 c["lens0"], c["slots"], SCAN_CHUNK,
+                                 *_SILU_ROWS)
             # the matrix-core passes keep their scratch states transposed
             S.lightning_combine(part, decay, state, c["off"], c["rows"],
                                 cu_seqlens, seq_lens, state_slots, mfma)
             if mfma:
-                S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 2)
+                S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 2,
+                                 *_SILU_ROWS)
             else:
                 S.lightning_scan(out, q, k, v, decay, part, c["cu"],
-                                 c["lens1"], c["slots"], SCAN_CHUNK)
+                                 c["lens1"], c["slots"], SCAN_CHUNK,
+                                 *_SILU_ROWS)
             return out
         S.lightning_scan(out, q, k, v, decay, state, cu_seqlens, seq_lens,
-                         state_slots, max_q_len)
+                         state_slots, max_q_len, *_SILU_ROWS)
         return out
     return ref.lightning_scan(q, k, v, decay, state, cu_seqlens, seq_lens,
                               state_slots)
@@ -830,3 +839,172 @@ def gelu_tanh(x):
         _native_seq().gelu_tanh(out, x)
         return out
     return ref.gelu_tanh(x)
+
+
+# ----------------------------------------------------------------------
+# Stream-residual blocks, window attention with pooled blocks, rotary
+# retention, clamped GLU, grouped routing (same extension, same rule).
+# ----------------------------------------------------------------------
+def stream_mix_norm(xs, y, y_bias, mix, out_w, in_w, norm_w, norm_b, eps):
+    """Residual kept as s weighted copies xs [s, T, C] fp32. With y: every
+    copy is rewritten from all old ones, new[t] = sum_s mix[s,t] old[s] +
+    out_w[t] (y + y_bias). With in_w: returns layer_norm(sum_s in_w[s]
+    new[s]) * norm_w + norm_b as fp32 [T, C] — the next sublayer's input,
+    produced by the same pass over the rows."""
+    if xs.is_cuda:
+        s, T, C = xs.shape
+        n = (torch.empty((T, C), dtype=torch.float32, device=xs.device)
+             if in_w is not None else None)
+        _native_seq().stream_mix_norm(xs, n, y, y_bias, mix, out_w, in_w,
+                                      norm_w, norm_b, eps)
+        return n
+    return ref.stream_mix_norm(xs, y, y_bias, mix, out_w, in_w, norm_w,
+                               norm_b, eps)
+
+
+def short_conv_residual(h, weight, state, cu_seqlens, seq_lens, state_slots,
+                        token_seq, out_dtype):
+    """h + causal depthwise conv of h over time (taps = weight.shape[1],
+    history of taps-1 rows per sequence in `state`), cast to out_dtype."""
+    if h.is_cuda:
+        out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+        _native_seq().short_conv_residual(out, h, weight, state, cu_seqlens,
+                                          seq_lens, state_slots, token_seq)
+        return out
+    return ref.short_conv_residual(h, weight, state, cu_seqlens, seq_lens,
+                                   state_slots, out_dtype)
+
+
+pool_slots_per_page = ref.pool_slots_per_page
+
+
+def kv_write_pooled(k, v, k_cache, v_cache, kp_cache, vp_cache, slot_mapping,
+                    positions, block_tables, token_seq, pool):
+    """Write the step's keys/values to their pages, then the mean key and
+    value of every block of `pool` positions this step completes into the
+    pooled caches (see ref.kv_write_pooled for the layout)."""
+    if k.is_cuda:
+        _native_seq().kv_write_pooled(k, v, k_cache, v_cache, kp_cache,
+                                      vp_cache, slot_mapping, positions,
+                                      block_tables, token_seq, pool)
+        return
+    ref.kv_write_pooled(k, v, k_cache, v_cache, kp_cache, vp_cache,
+                        slot_mapping, positions, block_tables, token_seq, pool)
+
+
+use_window_mfma = True  # tests switch it off to compare both paths
+
+
+def attention_window_pool(q, k_cache, v_cache, kp_cache, vp_cache,
+                          block_tables, seq_lens, cu_seqlens, token_seq,
+                          scale, window, pool, out, out_scale=1.0,
+                          max_q_len=0):
+    """Sliding-window softmax attention whose rows also see one pooled
+    key/value per block of `pool` positions older than every key of the
+    window (ref.attention_window_pool). Writes out [T, H, V] (may be a
+    column slice of a wider row), scaled by out_scale."""
+    if q.is_cuda:
+        S = _native_seq()
+        if not (use_window_mfma and q.dtype == torch.bfloat16 and max_q_len > 1
+                and S.attention_window_pool_mfma(
+                    out, q, k_cache, v_cache, kp_cache, vp_cache, block_tables,
+                    seq_lens, cu_seqlens, token_seq, scale, window, pool,
+                    out_scale)):
+            S.attention_window_pool(
+                out, q, k_cache, v_cache, kp_cache, vp_cache, block_tables,
+                seq_lens, cu_seqlens, token_seq, scale, window, pool,
+                out_scale)
+        return out
+    return ref.attention_window_pool(q, k_cache, v_cache, kp_cache, vp_cache,
+                                     block_tables, seq_lens, cu_seqlens,
+                                     scale, window, pool, out, out_scale)
+
+
+def retention_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
+                   positions, inv_freq, interleaved, k_scale, max_q_len=0,
+                   chunks=None):
+    """The lightning kernels on plain rows: q and k are turned by their
+    position (first 2*len(inv_freq) dims) and k scaled as they are loaded,
+    nothing is activated. chunks: chunk-parallel prefill as lightning_scan."""
+    if q.is_cuda:
+        T, H, D = q.shape
+        V = v.shape[2]
+        S = _native_seq()
+        out = torch.empty((T, H, V), dtype=torch.float32, device=q.device)
+        rot = (positions, inv_freq, bool(interleaved), float(k_scale))
+        if chunks is not None and max_q_len > SCAN_CHUNK:
+            c = chunks
+            part = torch.empty((c["n"], H, D, V), dtype=torch.float32,
+                               device=q.device)
+            mfma = (q.dtype == torch.bfloat16 and use_lightning_mfma
+                    and S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 1,
+                                         *rot))
+            if not mfma:
+                S.lightning_scan(out, q, k, v, decay, part, c["cu"],
+                                 c["lens0"], c["slots"], SCAN_CHUNK, *rot)
+            S.lightning_combine(part, decay, state, c["off"], c["rows"],
+                                cu_seqlens, seq_lens, state_slots, mfma)
+            if mfma:
+                S.lightning_mfma(out, part, q, k, v, decay, c["cu"], 2, *rot)
+            else:
+                S.lightning_scan(out, q, k, v, decay, part, c["cu"],
+                                 c["lens1"], c["slots"], SCAN_CHUNK, *rot)
+            return out
+        S.lightning_scan(out, q, k, v, decay, state, cu_seqlens, seq_lens,
+                         state_slots, max_q_len, *rot)
+        return out
+    return ref.retention_scan(q, k, v, decay, state, cu_seqlens, seq_lens,
+                              state_slots, positions, inv_freq, interleaved,
+                              k_scale)
+
+
+def head_norm_gate(o, gate, eps, heads, out, out_scale=1.0):
+    """Per-head unit RMS of o [T, heads*V] fp32, times silu(gate), times
+    out_scale, into out (may be a column slice of a wider row)."""
+    if o.is_cuda:
+        _native_seq().head_norm_gate(out, o, gate, eps, heads, out_scale)
+        return out
+    return ref.head_norm_gate(o, gate, eps, heads, out, out_scale)
+
+
+def glu_act(gu, kind, limit=0.0, alpha=1.0):
+    """[gate | up] rows -> activated rows (ref.glu_act)."""
+    if gu.is_cuda:
+        F_ = gu.shape[-1] // 2
+        out = torch.empty((gu.shape[0], F_), dtype=gu.dtype, device=gu.device)
+        _native_seq().glu_act(out, gu, 0 if kind == "swiglu" else 1,
+                              float(limit), float(alpha))
+        return out
+    return ref.glu_act(gu, kind, limit, alpha)
+
+
+def moe_route_grouped(logits, top, groups, keep):
+    """Group-limited routing: (weights [T, top] fp32, ids [T, top] int32)."""
+    if logits.is_cuda:
+        T = logits.shape[0]
+        w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+        ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+        _native_seq().moe_route_grouped(w, ids, logits.contiguous(), top,
+                                        groups, keep)
+        return w, ids
+    return ref.moe_route_grouped(logits, top, groups, keep)
+
+
+def moe_mix_seq(y, weights, ids):
+    """moe_mix for callers of the sequence-state extension (any float
+    dtype of y)."""
+    if y.is_cuda:
+        El, T, H = y.shape
+        out = torch.empty(T, H, dtype=y.dtype, device=y.device)
+        _native_seq().moe_mix(out, y.contiguous(), weights, ids)
+        return out
+    return ref.moe_mix(y, weights, ids, 0)
+
+
+def moe_mix_rows_seq(y, weights, rows):
+    if y.is_cuda:
+        T, k = weights.shape
+        out = torch.empty(T, y.shape[1], dtype=y.dtype, device=y.device)
+        _native_seq().moe_mix_rows(out, y.contiguous(), weights, rows)
+        return out
+    return ref.moe_mix_rows(y, weights, rows)

@@ -48,6 +48,10 @@ SEQ_SOURCES = [
     os.path.join(CSRC, "seq_lightning.hip"),
     os.path.join(CSRC, "seq_lightning_mfma.hip"),
     os.path.join(CSRC, "seq_mamba.hip"),
+    os.path.join(CSRC, "seq_stream.hip"),
+    os.path.join(CSRC, "seq_window.hip"),
+    os.path.join(CSRC, "seq_window_mfma.hip"),
+    os.path.join(CSRC, "seq_moe.hip"),
 ]
 
 EXTENSIONS = {EXT_NAME: SOURCES, SEQ_EXT_NAME: SEQ_SOURCES}

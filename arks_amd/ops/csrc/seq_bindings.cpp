@@ -42,7 +42,9 @@ int arks_seq_lightning_scan(void* out, const void* q, const void* k,
                             int64_t ldv, const void* decay, void* state,
                             const void* cu, const void* seq_lens,
                             const void* slots, int S, int H, int D, int V,
-                            int act_f32, hipStream_t stream);
+                            int act_f32, int mode, const void* positions,
+                            const void* freq, int n_rot, int interleaved,
+                            float k_scale, hipStream_t stream);
 int arks_seq_causal_conv_silu(void* out, const void* x, int64_t ldx,
                               const void* w, const void* w_t, const void* bias,
                               void* state,
@@ -65,7 +67,61 @@ int arks_seq_lightning_mfma(void* out, void* part, const void* q, const void* k,
                             const void* v, int64_t ldq, int64_t ldk,
                             int64_t ldv, const void* decay, const void* cu,
                             int chunks, int H, int D, int V, int pass,
+                            int mode, const void* positions, const void* freq,
+                            int n_rot, int interleaved, float k_scale,
                             hipStream_t stream);
+int arks_seq_stream_mix_norm(void* xs, void* n_out, const void* y, int64_t ldy,
+                             const void* y_bias, const void* mix,
+                             const void* out_w, const void* in_w,
+                             const void* norm_w, const void* norm_b, float eps,
+                             int S, int64_t T, int C, int act_f32,
+                             hipStream_t stream);
+int arks_seq_short_conv_residual(void* out, const void* h, const void* w,
+                                 void* state, const void* cu,
+                                 const void* seq_lens, const void* slots,
+                                 const void* token_seq, int T, int S, int C,
+                                 int taps, int act_f32, hipStream_t stream);
+void arks_seq_head_norm_gate(void* out, int64_t ldo, const void* o,
+                             const void* gate, int64_t ldg, float eps, int T,
+                             int H, int V, float out_scale, int act_f32,
+                             hipStream_t stream);
+void arks_seq_glu_act(void* out, const void* gu, int64_t ldg, int64_t rows,
+                      int F, int mode, float limit, float alpha, int act_f32,
+                      hipStream_t stream);
+void arks_seq_kv_write_pooled(const void* k, const void* v, int64_t ldk,
+                              int64_t ldv, void* k_cache, void* v_cache,
+                              void* kp_cache, void* vp_cache,
+                              const void* slot_mapping, const void* positions,
+                              const void* block_tables, const void* token_seq,
+                              int T, int max_blocks, int G, int D, int V,
+                              int bs, int pool, int spp, int act_f32,
+                              hipStream_t stream);
+int arks_seq_attn_window_pool(void* out, int64_t ldo, const void* q,
+                              int64_t ldq, const void* k_cache,
+                              const void* v_cache, const void* kp_cache,
+                              const void* vp_cache, const void* block_tables,
+                              const void* seq_lens, const void* cu,
+                              const void* token_seq, float scale, int window,
+                              int pool, int spp, float out_scale, int T, int H,
+                              int G, int D, int V, int bs, int max_blocks,
+                              int act_f32, hipStream_t stream);
+int arks_seq_attn_window_pool_mfma(void* out, int64_t ldo, const void* q,
+                                   int64_t ldq, const void* k_cache,
+                                   const void* v_cache, const void* kp_cache,
+                                   const void* vp_cache,
+                                   const void* block_tables,
+                                   const void* seq_lens, const void* cu,
+                                   const void* token_seq, float scale,
+                                   int window, int pool, int spp,
+                                   float out_scale, int T, int H, int G, int D,
+                                   int V, int bs, int max_blocks,
+                                   int num_seqs, hipStream_t stream);
+int arks_seq_moe_route_grouped(void* weights, void* ids, const void* logits,
+                               int T, int E, int top, int groups, int keep,
+                               hipStream_t stream);
+void arks_seq_moe_mix_rows(void* out, const void* y, const void* weights,
+                           const void* rows, int T, int H, int k, int dense,
+                           int act_f32, hipStream_t stream);
 void arks_seq_lightning_combine(void* part, const void* decay, void* state,
                                 const void* chunk_off, const void* chunk_rows,
                                 const void* cu, const void* seq_lens,
@@ -336,10 +392,38 @@ void unrotate_rows(Tensor out, Tensor positions, Tensor freq_v,
   TORCH_CHECK(rc == 0, "more rotary pairs than the kernel's table holds");
 }
 
+// Input convention of the lightning kernels: without positions, rows pass
+// through silu (mode 0); with positions, plain rows whose q and k are turned
+// over their first 2 * freq.numel() dims (mode 1; freq may be absent).
+struct RotArgs {
+  int mode, n_rot;
+  const void* positions;
+  const void* freq;
+};
+
+RotArgs rot_args(const OptTensor& positions, const OptTensor& freq, int64_t T,
+                 int64_t D) {
+  RotArgs r{0, 0, nullptr, nullptr};
+  if (!positions.has_value()) return r;
+  check_i64(*positions, "positions");
+  TORCH_CHECK(positions->numel() == T, "one position per row");
+  r.mode = 1;
+  r.positions = positions->data_ptr();
+  if (freq.has_value() && freq->numel() > 0) {
+    check_f32(*freq, "rotary frequencies");
+    TORCH_CHECK(2 * freq->numel() <= D, "more rotary dims than the head has");
+    r.n_rot = (int)freq->numel();
+    r.freq = freq->data_ptr();
+  }
+  return r;
+}
+
 void lightning_scan(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
                     Tensor state, Tensor cu, Tensor seq_lens, Tensor slots,
-                    int64_t max_q_len) {
+                    int64_t max_q_len, OptTensor positions, OptTensor freq,
+                    bool interleaved, double k_scale) {
   const int f32 = act_flag(q, "q");
+  const RotArgs rot = rot_args(positions, freq, q.size(0), q.size(2));
   const int T = q.size(0), H = q.size(1), D = q.size(2), V = v.size(2);
   TORCH_CHECK(k.scalar_type() == q.scalar_type() &&
               v.scalar_type() == q.scalar_type());
@@ -357,7 +441,8 @@ void lightning_scan(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
       out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
       head_row_stride(q, "q"), head_row_stride(k, "k"), head_row_stride(v, "v"),
       decay.data_ptr(), state.data_ptr(), cu.data_ptr(), seq_lens.data_ptr(),
-      slots.data_ptr(), m.S, H, D, V, f32, current_stream());
+      slots.data_ptr(), m.S, H, D, V, f32, rot.mode, rot.positions, rot.freq,
+      rot.n_rot, interleaved ? 1 : 0, (float)k_scale, current_stream());
   TORCH_CHECK(rc == 0, "lightning head size beyond the kernel's limit (", D, ")");
 }
 
@@ -476,7 +561,9 @@ void scan_combine(Tensor part, Tensor dsum, Tensor A, Tensor state,
 // reads chunk start states from part and writes out. False: no kernel for
 // these head sizes (the caller runs the general kernel).
 bool lightning_mfma(Tensor out, Tensor part, Tensor q, Tensor k, Tensor v,
-                    Tensor decay, Tensor cu, int64_t pass) {
+                    Tensor decay, Tensor cu, int64_t pass, OptTensor positions,
+                    OptTensor freq, bool interleaved, double k_scale) {
+  const RotArgs rot = rot_args(positions, freq, q.size(0), q.size(2));
   TORCH_CHECK(q.is_cuda() && q.scalar_type() == torch::kBFloat16 &&
               k.scalar_type() == torch::kBFloat16 &&
               v.scalar_type() == torch::kBFloat16, "bf16 rows only");
@@ -496,7 +583,8 @@ bool lightning_mfma(Tensor out, Tensor part, Tensor q, Tensor k, Tensor v,
              out.data_ptr(), part.data_ptr(), q.data_ptr(), k.data_ptr(),
              v.data_ptr(), head_row_stride(q, "q"), head_row_stride(k, "k"),
              head_row_stride(v, "v"), decay.data_ptr(), cu.data_ptr(), chunks,
-             H, D, V, (int)pass, current_stream()) == 0;
+             H, D, V, (int)pass, rot.mode, rot.positions, rot.freq, rot.n_rot,
+             interleaved ? 1 : 0, (float)k_scale, current_stream()) == 0;
 }
 
 void lightning_combine(Tensor part, Tensor decay, Tensor state,
@@ -523,9 +611,260 @@ void lightning_combine(Tensor part, Tensor decay, Tensor state,
                              V, transposed ? 1 : 0, current_stream());
 }
 
+// ---- stream arrangement, window/pool attention, grouped routing
+
+void stream_mix_norm(Tensor xs, OptTensor n_out, OptTensor y, OptTensor y_bias,
+                     OptTensor mix, OptTensor out_w, OptTensor in_w,
+                     OptTensor norm_w, OptTensor norm_b, double eps) {
+  check_f32(xs, "xs");
+  TORCH_CHECK(xs.dim() == 3, "xs must be [streams, T, C]");
+  const int S = xs.size(0), C = xs.size(2);
+  const int64_t T = xs.size(1);
+  int f32 = 1;
+  int64_t ldy = 0;
+  if (y.has_value()) {
+    f32 = act_flag(*y, "y");
+    TORCH_CHECK(y->size(0) == T && y->size(1) == C);
+    ldy = row_stride(*y, "y");
+    TORCH_CHECK(mix.has_value() && out_w.has_value());
+    check_f32(*mix, "mix");
+    check_f32(*out_w, "out weights");
+    TORCH_CHECK(mix->numel() == S * S && out_w->numel() == S);
+    if (y_bias.has_value()) {
+      check_f32(*y_bias, "y bias");
+      TORCH_CHECK(y_bias->numel() == C);
+    }
+  }
+  if (in_w.has_value()) {
+    check_f32(*in_w, "in weights");
+    check_f32(*norm_w, "norm weight");
+    check_f32(*norm_b, "norm bias");
+    check_f32(*n_out, "norm output");
+    TORCH_CHECK(in_w->numel() == S && norm_w->numel() == C &&
+                norm_b->numel() == C && n_out->size(0) == T &&
+                n_out->size(1) == C);
+  }
+  const int rc = arks_seq_stream_mix_norm(
+      xs.data_ptr(), in_w.has_value() ? n_out->data_ptr() : nullptr,
+      y.has_value() ? y->data_ptr() : nullptr, ldy,
+      y.has_value() && y_bias.has_value() ? y_bias->data_ptr() : nullptr,
+      y.has_value() ? mix->data_ptr() : nullptr,
+      y.has_value() ? out_w->data_ptr() : nullptr,
+      in_w.has_value() ? in_w->data_ptr() : nullptr,
+      in_w.has_value() ? norm_w->data_ptr() : nullptr,
+      in_w.has_value() ? norm_b->data_ptr() : nullptr, (float)eps, S, T, C,
+      f32, current_stream());
+  TORCH_CHECK(rc == 0, "more residual copies or a wider row than the kernel holds");
+}
+
+void short_conv_residual(Tensor out, Tensor h, Tensor w, OptTensor state,
+                         Tensor cu, Tensor seq_lens, Tensor slots,
+                         Tensor token_seq) {
+  check_f32(h, "h");
+  check_f32(w, "conv weight");
+  const int f32 = act_flag(out, "out");
+  const int T = h.size(0), C = h.size(1), taps = w.size(1);
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == h.sizes());
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C && taps >= 1);
+  const SeqMeta m = check_meta(cu, seq_lens, &slots, &token_seq, T);
+  if (taps > 1) {
+    TORCH_CHECK(state.has_value(), "a conv with history needs its state");
+    check_f32(*state, "conv state");
+    TORCH_CHECK(state->dim() == 3 && state->size(1) == taps - 1 &&
+                state->size(2) == C, "state must be [slots, taps-1, C]");
+  }
+  const int rc = arks_seq_short_conv_residual(
+      out.data_ptr(), h.data_ptr(), w.data_ptr(),
+      taps > 1 ? state->data_ptr() : nullptr, cu.data_ptr(),
+      seq_lens.data_ptr(), slots.data_ptr(), token_seq.data_ptr(), T, m.S, C,
+      taps, f32, current_stream());
+  TORCH_CHECK(rc == 0, "more conv taps than the kernel holds");
+}
+
+void head_norm_gate(Tensor out, Tensor o, Tensor gate, double eps,
+                    int64_t heads, double out_scale) {
+  check_f32(o, "o");
+  const int f32 = act_flag(out, "out");
+  TORCH_CHECK(o.dim() == 2 && o.size(1) % heads == 0);
+  TORCH_CHECK(gate.scalar_type() == out.scalar_type() &&
+              gate.sizes() == o.sizes() && out.sizes() == o.sizes());
+  arks_seq_head_norm_gate(out.data_ptr(), row_stride(out, "out"), o.data_ptr(),
+                          gate.data_ptr(), row_stride(gate, "gate"),
+                          (float)eps, o.size(0), heads, o.size(1) / heads,
+                          (float)out_scale, f32, current_stream());
+}
+
+void glu_act(Tensor out, Tensor gu, int64_t mode, double limit, double alpha) {
+  const int f32 = act_flag(gu, "gate|up");
+  TORCH_CHECK(gu.dim() == 2 && gu.size(1) % 2 == 0);
+  const int F = gu.size(1) / 2;
+  TORCH_CHECK(out.scalar_type() == gu.scalar_type() && out.is_contiguous() &&
+              out.size(0) == gu.size(0) && out.size(1) == F);
+  arks_seq_glu_act(out.data_ptr(), gu.data_ptr(), row_stride(gu, "gate|up"),
+                   gu.size(0), F, (int)mode, (float)limit, (float)alpha, f32,
+                   current_stream());
+}
+
+struct WindowShapes {
+  int T, H, G, D, V, bs, spp, max_blocks, f32;
+};
+
+WindowShapes check_window(const Tensor& q, const Tensor& k_cache,
+                          const Tensor& v_cache, const Tensor& kp,
+                          const Tensor& vp, const Tensor& block_tables,
+                          int64_t pool) {
+  WindowShapes w;
+  w.f32 = act_flag(q, "q");
+  TORCH_CHECK(q.dim() == 3);
+  w.T = q.size(0); w.H = q.size(1); w.D = q.size(2);
+  for (const Tensor* c : {&k_cache, &v_cache, &kp, &vp})
+    TORCH_CHECK(c->is_cuda() && c->is_contiguous() && c->dim() == 4 &&
+                c->scalar_type() == q.scalar_type(),
+                "caches must be contiguous [pages, G, n, dim] of q's dtype");
+  w.G = k_cache.size(1); w.bs = k_cache.size(2); w.V = v_cache.size(3);
+  w.spp = kp.size(2);
+  TORCH_CHECK(pool >= 1 && w.spp == (w.bs - 1) / pool + 1,
+              "pooled cache does not fit the pool size");
+  TORCH_CHECK(k_cache.size(3) == w.D && kp.size(3) == w.D &&
+              vp.size(3) == w.V && v_cache.size(1) == w.G &&
+              kp.size(1) == w.G && vp.size(1) == w.G &&
+              v_cache.size(2) == w.bs && vp.size(2) == w.spp &&
+              kp.size(0) == k_cache.size(0) && vp.size(0) == k_cache.size(0) &&
+              v_cache.size(0) == k_cache.size(0) && w.H % w.G == 0);
+  check_i32(block_tables, "block_tables");
+  TORCH_CHECK(block_tables.dim() == 2);
+  w.max_blocks = block_tables.size(1);
+  return w;
+}
+
+void kv_write_pooled(Tensor k, Tensor v, Tensor k_cache, Tensor v_cache,
+                     Tensor kp, Tensor vp, Tensor slot_mapping,
+                     Tensor positions, Tensor block_tables, Tensor token_seq,
+                     int64_t pool) {
+  const int f32 = act_flag(k, "k");
+  TORCH_CHECK(k.dim() == 3 && v.dim() == 3 &&
+              v.scalar_type() == k.scalar_type());
+  for (const Tensor* c : {&k_cache, &v_cache, &kp, &vp})
+    TORCH_CHECK(c->is_cuda() && c->is_contiguous() && c->dim() == 4 &&
+                c->scalar_type() == k.scalar_type());
+  const int T = k.size(0), G = k.size(1), D = k.size(2), V = v.size(2);
+  const int bs = k_cache.size(2), spp = kp.size(2);
+  TORCH_CHECK(v.size(0) == T && v.size(1) == G && k_cache.size(1) == G &&
+              k_cache.size(3) == D && v_cache.size(1) == G &&
+              v_cache.size(2) == bs && v_cache.size(3) == V &&
+              kp.size(1) == G && kp.size(3) == D && vp.size(1) == G &&
+              vp.size(2) == spp && vp.size(3) == V);
+  TORCH_CHECK(pool >= 1 && spp == (bs - 1) / pool + 1);
+  check_i64(slot_mapping, "slot_mapping");
+  check_i64(positions, "positions");
+  check_i32(block_tables, "block_tables");
+  check_i32(token_seq, "token_seq");
+  TORCH_CHECK(slot_mapping.numel() == T && positions.numel() == T &&
+              token_seq.numel() == T && block_tables.dim() == 2);
+  arks_seq_kv_write_pooled(
+      k.data_ptr(), v.data_ptr(), head_row_stride(k, "k"),
+      head_row_stride(v, "v"), k_cache.data_ptr(), v_cache.data_ptr(),
+      kp.data_ptr(), vp.data_ptr(), slot_mapping.data_ptr(),
+      positions.data_ptr(), block_tables.data_ptr(), token_seq.data_ptr(), T,
+      (int)block_tables.size(1), G, D, V, bs, (int)pool, spp, f32,
+      current_stream());
+}
+
+void attention_window_pool(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                           Tensor kp, Tensor vp, Tensor block_tables,
+                           Tensor seq_lens, Tensor cu, Tensor token_seq,
+                           double scale, int64_t window, int64_t pool,
+                           double out_scale) {
+  const WindowShapes w = check_window(q, k_cache, v_cache, kp, vp,
+                                      block_tables, pool);
+  TORCH_CHECK(out.scalar_type() == q.scalar_type() && out.dim() == 3 &&
+              out.size(0) == w.T && out.size(1) == w.H && out.size(2) == w.V);
+  check_meta(cu, seq_lens, nullptr, &token_seq, w.T);
+  TORCH_CHECK(block_tables.size(0) == seq_lens.numel() && window >= 1);
+  const int rc = arks_seq_attn_window_pool(
+      out.data_ptr(), head_row_stride(out, "out"), q.data_ptr(),
+      head_row_stride(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(),
+      kp.data_ptr(), vp.data_ptr(), block_tables.data_ptr(),
+      seq_lens.data_ptr(), cu.data_ptr(), token_seq.data_ptr(), (float)scale,
+      (int)window, (int)pool, w.spp, (float)out_scale, w.T, w.H, w.G, w.D, w.V,
+      w.bs, w.max_blocks, w.f32, current_stream());
+  TORCH_CHECK(rc == 0, "head size beyond the kernel's limit");
+}
+
+// The matrix-core kernel; false: not built for these sizes (the caller
+// runs the general kernel).
+bool attention_window_pool_mfma(Tensor out, Tensor q, Tensor k_cache,
+                                Tensor v_cache, Tensor kp, Tensor vp,
+                                Tensor block_tables, Tensor seq_lens, Tensor cu,
+                                Tensor token_seq, double scale, int64_t window,
+                                int64_t pool, double out_scale) {
+  const WindowShapes w = check_window(q, k_cache, v_cache, kp, vp,
+                                      block_tables, pool);
+  TORCH_CHECK(w.f32 == 0, "bf16 rows only");
+  TORCH_CHECK(out.scalar_type() == q.scalar_type() && out.dim() == 3 &&
+              out.size(0) == w.T && out.size(1) == w.H && out.size(2) == w.V);
+  check_meta(cu, seq_lens, nullptr, &token_seq, w.T);
+  TORCH_CHECK(block_tables.size(0) == seq_lens.numel() && window >= 1);
+  return arks_seq_attn_window_pool_mfma(
+             out.data_ptr(), head_row_stride(out, "out"), q.data_ptr(),
+             head_row_stride(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(),
+             kp.data_ptr(), vp.data_ptr(), block_tables.data_ptr(),
+             seq_lens.data_ptr(), cu.data_ptr(), token_seq.data_ptr(),
+             (float)scale, (int)window, (int)pool, w.spp, (float)out_scale,
+             w.T, w.H, w.G, w.D, w.V, w.bs, w.max_blocks,
+             (int)seq_lens.numel(), current_stream()) == 0;
+}
+
+void moe_route_grouped(Tensor weights, Tensor ids, Tensor logits, int64_t top,
+                       int64_t groups, int64_t keep) {
+  check_f32(logits, "router logits");
+  check_f32(weights, "weights");
+  check_i32(ids, "ids");
+  const int T = logits.size(0), E = logits.size(1);
+  TORCH_CHECK(weights.size(0) == T && weights.size(1) == top &&
+              ids.size(0) == T && ids.size(1) == top);
+  const int rc = arks_seq_moe_route_grouped(
+      weights.data_ptr(), ids.data_ptr(), logits.data_ptr(), T, E, (int)top,
+      (int)groups, (int)keep, current_stream());
+  TORCH_CHECK(rc == 0, "routing sizes the kernel does not hold");
+}
+
+void moe_mix_common(Tensor out, Tensor y, Tensor weights, Tensor rows,
+                    int dense) {
+  const int f32 = act_flag(y, "y");
+  check_f32(weights, "weights");
+  check_i32(rows, "rows");
+  TORCH_CHECK(y.is_contiguous() && out.is_contiguous() &&
+              out.scalar_type() == y.scalar_type());
+  const int T = weights.size(0), k = weights.size(1), H = out.size(1);
+  TORCH_CHECK(out.size(0) == T && rows.numel() == (int64_t)T * k &&
+              y.size(-1) == H);
+  if (dense) TORCH_CHECK(y.dim() == 3 && y.size(1) == T);
+  arks_seq_moe_mix_rows(out.data_ptr(), y.data_ptr(), weights.data_ptr(),
+                        rows.data_ptr(), T, H, k, dense, f32, current_stream());
+}
+
+void moe_mix(Tensor out, Tensor y, Tensor weights, Tensor ids) {
+  moe_mix_common(out, y, weights, ids, 1);
+}
+
+void moe_mix_rows(Tensor out, Tensor y, Tensor weights, Tensor rows) {
+  moe_mix_common(out, y, weights, rows, 0);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("stream_mix_norm", &stream_mix_norm);
+  m.def("short_conv_residual", &short_conv_residual);
+  m.def("head_norm_gate", &head_norm_gate);
+  m.def("glu_act", &glu_act);
+  m.def("kv_write_pooled", &kv_write_pooled);
+  m.def("attention_window_pool", &attention_window_pool);
+  m.def("attention_window_pool_mfma", &attention_window_pool_mfma);
+  m.def("moe_route_grouped", &moe_route_grouped);
+  m.def("moe_mix", &moe_mix);
+  m.def("moe_mix_rows", &moe_mix_rows);
   def_paged_attention(m);
   m.def("unrotate_rows", &unrotate_rows);
   m.def("token_shift", &token_shift);

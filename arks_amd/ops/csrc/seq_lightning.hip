@@ -3,6 +3,11 @@
 // S is a [D x V] fp32 matrix per head and sequence, kept in a slot-addressed
 // state tensor between steps.
 //
+// Two input conventions (template MODE): 0 — q, k and v pass through silu;
+// 1 — plain rows, q and k turned by their position over their first 2*n_rot
+// dims (pairs (2i, 2i+1) when interleaved, (i, i+n_rot) otherwise; angle =
+// position * freq[i], fp32) and k multiplied by k_scale after that.
+//
 // General kernel: one wave per (sequence, head, 64 value columns); lane c
 // owns column c of S in registers and walks the sequence's rows in order.
 // The row's silu(q), silu(k) are staged in LDS once per row for all lanes.
@@ -10,13 +15,31 @@
 
 namespace arks {
 
-template <typename AT, int DMAX>
+// Element d of a head's q or k row turned by `pos` (MODE 1 loads).
+template <typename AT>
+__device__ __forceinline__ float rotated_ld(const AT* row, int d, float pos,
+                                            const float* freq, int n_rot,
+                                            int interleaved) {
+  const float x = Act<AT>::ld(row + d);
+  if (d >= 2 * n_rot) return x;
+  const int i = interleaved ? d >> 1 : (d < n_rot ? d : d - n_rot);
+  const bool first = interleaved ? !(d & 1) : d < n_rot;
+  const int dp = interleaved ? d ^ 1 : (first ? d + n_rot : d - n_rot);
+  const float y = Act<AT>::ld(row + dp);
+  float sn, cs;
+  sincosf(pos * freq[i], &sn, &cs);
+  return first ? x * cs - y * sn : x * cs + y * sn;
+}
+
+template <typename AT, int DMAX, int MODE>
 __global__ __launch_bounds__(64) void lightning_scan_kernel(
     float* __restrict__ out, const AT* __restrict__ q, const AT* __restrict__ k,
     const AT* __restrict__ v, int64_t ldq, int64_t ldk, int64_t ldv,
     const float* __restrict__ decay, float* __restrict__ state,
     const int* __restrict__ cu, const int* __restrict__ seq_lens,
-    const int* __restrict__ slots, int H, int D, int V) {
+    const int* __restrict__ slots, int H, int D, int V,
+    const int64_t* __restrict__ positions, const float* __restrict__ freq,
+    int n_rot, int interleaved, float k_scale) {
   __shared__ float q_s[2][DMAX];
   __shared__ float k_s[2][DMAX];
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -36,12 +59,25 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(
   for (int r = 0; r < rows; ++r) {
     const int t = a + r;
     const int buf = r & 1;  // double buffer: one barrier per row
-    for (int d = lane; d < D; d += 64) {
-      q_s[buf][d] = silu_f(Act<AT>::ld(q + (int64_t)t * ldq + (int64_t)h * D + d));
-      k_s[buf][d] = silu_f(Act<AT>::ld(k + (int64_t)t * ldk + (int64_t)h * D + d));
+    if (MODE == 0) {
+      for (int d = lane; d < D; d += 64) {
+        q_s[buf][d] = silu_f(Act<AT>::ld(q + (int64_t)t * ldq + (int64_t)h * D + d));
+        k_s[buf][d] = silu_f(Act<AT>::ld(k + (int64_t)t * ldk + (int64_t)h * D + d));
+      }
+    } else {
+      const float pos = (float)positions[t];
+      for (int d = lane; d < D; d += 64) {
+        q_s[buf][d] = rotated_ld<AT>(q + (int64_t)t * ldq + (int64_t)h * D, d,
+                                     pos, freq, n_rot, interleaved);
+        k_s[buf][d] = k_scale * rotated_ld<AT>(k + (int64_t)t * ldk + (int64_t)h * D,
+                                               d, pos, freq, n_rot, interleaved);
+      }
     }
-    const float vv =
-        live ? silu_f(Act<AT>::ld(v + (int64_t)t * ldv + (int64_t)h * V + col)) : 0.f;
+    float vv = 0.f;
+    if (live) {
+      vv = Act<AT>::ld(v + (int64_t)t * ldv + (int64_t)h * V + col);
+      if (MODE == 0) vv = silu_f(vv);
+    }
     __syncthreads();
     float o = 0.f;
 #pragma unroll
@@ -116,18 +152,21 @@ extern "C" void arks_seq_lightning_combine(void* part, const void* decay,
                      D, V, transposed);
 }
 
-template <typename AT>
+template <typename AT, int MODE>
 static int launch_lightning(float* out, const void* q, const void* k,
                             const void* v, int64_t ldq, int64_t ldk,
                             int64_t ldv, const float* decay, float* state,
                             const int* cu, const int* seq_lens,
                             const int* slots, int S, int H, int D, int V,
+                            const int64_t* positions, const float* freq,
+                            int n_rot, int interleaved, float k_scale,
                             hipStream_t stream) {
   dim3 grid(S, H, (V + 63) / 64), block(64);
 #define LL(DM)                                                                 \
-  hipLaunchKernelGGL((lightning_scan_kernel<AT, DM>), grid, block, 0, stream,  \
-                     out, (const AT*)q, (const AT*)k, (const AT*)v, ldq, ldk,  \
-                     ldv, decay, state, cu, seq_lens, slots, H, D, V)
+  hipLaunchKernelGGL((lightning_scan_kernel<AT, DM, MODE>), grid, block, 0,    \
+                     stream, out, (const AT*)q, (const AT*)k, (const AT*)v,    \
+                     ldq, ldk, ldv, decay, state, cu, seq_lens, slots, H, D,   \
+                     V, positions, freq, n_rot, interleaved, k_scale)
   if (D <= 16) LL(16);
   else if (D <= 32) LL(32);
   else if (D <= 64) LL(64);
@@ -142,12 +181,18 @@ extern "C" int arks_seq_lightning_scan(
     void* out, const void* q, const void* k, const void* v, int64_t ldq,
     int64_t ldk, int64_t ldv, const void* decay, void* state, const void* cu,
     const void* seq_lens, const void* slots, int S, int H, int D, int V,
-    int act_f32, hipStream_t stream) {
+    int act_f32, int mode, const void* positions, const void* freq, int n_rot,
+    int interleaved, float k_scale, hipStream_t stream) {
   if (S == 0) return 0;
   int rc = 0;
-  SEQ_DISPATCH_ACT(act_f32, rc = launch_lightning<AT>(
-      (float*)out, q, k, v, ldq, ldk, ldv, (const float*)decay, (float*)state,
-      (const int*)cu, (const int*)seq_lens, (const int*)slots, S, H, D, V,
-      stream));
+#define LS(MODE)                                                              \
+  SEQ_DISPATCH_ACT(act_f32, (rc = launch_lightning<AT, MODE>(                 \
+      (float*)out, q, k, v, ldq, ldk, ldv, (const float*)decay, (float*)state, \
+      (const int*)cu, (const int*)seq_lens, (const int*)slots, S, H, D, V,    \
+      (const int64_t*)positions, (const float*)freq, n_rot, interleaved,      \
+      k_scale, stream)))
+  if (mode == 0) LS(0);
+  else LS(1);
+#undef LS
   return rc;
 }

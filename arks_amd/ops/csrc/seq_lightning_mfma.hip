@@ -9,8 +9,9 @@
 // `part` holds each state TRANSPOSED ([v][d]): pass 2 then reads its state
 // operand (k = d contiguous) straight from global memory, and the combine
 // step between the passes is elementwise, so it does not care.
-// q, k, v are silu'd in fp32 on the way into LDS and rounded to bf16 for
-// v_mfma_f32_16x16x32_bf16. Every fp32 quantity that meets a matrix
+// q, k, v are silu'd (MODE 0), or q and k turned by their position and k
+// scaled (MODE 1, see seq_lightning.hip), in fp32 on the way into LDS and
+// rounded to bf16 for v_mfma_f32_16x16x32_bf16. Every fp32 quantity that meets a matrix
 // operand — the decayed keys of pass 1, the decayed score matrix and the
 // fp32 state of pass 2 — is split into a bf16 high and low part and
 // multiplied twice, so decays, scores and state keep ~16 mantissa bits
@@ -24,6 +25,30 @@
 #include "seq_common.h"
 
 namespace arks {
+
+struct LmRot {  // MODE 1 input transform
+  const int64_t* positions;
+  const float* freq;
+  int n_rot, interleaved;
+  float k_scale;
+};
+
+// Element d of head row `row` (bf16): silu (MODE 0) or position turn.
+template <int MODE>
+__device__ __forceinline__ float lm_load(const bf16* row, int d, int64_t t,
+                                         const LmRot& rot) {
+  const float x = bf16_bits_to_float(row[d]);
+  if (MODE == 0) return silu_f(x);
+  if (d >= 2 * rot.n_rot) return x;
+  const int n = rot.n_rot;
+  const int i = rot.interleaved ? d >> 1 : (d < n ? d : d - n);
+  const bool first = rot.interleaved ? !(d & 1) : d < n;
+  const int dp = rot.interleaved ? d ^ 1 : (first ? d + n : d - n);
+  const float y = bf16_bits_to_float(row[dp]);
+  float sn, cs;
+  sincosf((float)rot.positions[t] * rot.freq[i], &sn, &cs);
+  return first ? x * cs - y * sn : x * cs + y * sn;
+}
 
 typedef __attribute__((ext_vector_type(8))) __bf16 lm_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float lm_f32x4;
@@ -59,12 +84,12 @@ __device__ __forceinline__ float decay_pow(float log2_decay, int e) {
 }
 
 // ---- pass 1: end state of each chunk scanned from zero
-template <int D, int V>
+template <int D, int V, int MODE>
 __global__ __launch_bounds__(256) void lightning_state_mfma_kernel(
     float* __restrict__ part,  // [chunks, H, V, D] (transposed states)
     const bf16* __restrict__ k, const bf16* __restrict__ v, int64_t ldk,
     int64_t ldv, const float* __restrict__ decay, const int* __restrict__ cu,
-    int H) {
+    int H, LmRot rot) {
   constexpr int LK = LM_ROWS + LM_PAD;
   extern __shared__ __attribute__((aligned(16))) unsigned char lm_smem[];
   bf16* kt_hi = reinterpret_cast<bf16*>(lm_smem);  // [D][LK]
@@ -78,15 +103,18 @@ __global__ __launch_bounds__(256) void lightning_state_mfma_kernel(
     const int j = i / D, d = i - j * D;
     float x = 0.f;
     if (j < n)
-      x = silu_f(bf16_bits_to_float(k[(int64_t)(row0 + j) * ldk + (int64_t)h * D + d])) *
-          decay_pow(l2, n - 1 - j);
+      x = lm_load<MODE>(k + (int64_t)(row0 + j) * ldk + (int64_t)h * D, d,
+                        row0 + j, rot) *
+          (MODE == 0 ? 1.f : rot.k_scale) * decay_pow(l2, n - 1 - j);
     split_bf16(x, kt_hi[d * LK + j], kt_lo[d * LK + j]);
   }
   for (int i = tid; i < LM_ROWS * V; i += 256) {
     const int j = i / V, c = i - j * V;
     float x = 0.f;
-    if (j < n)
-      x = silu_f(bf16_bits_to_float(v[(int64_t)(row0 + j) * ldv + (int64_t)h * V + c]));
+    if (j < n) {
+      x = bf16_bits_to_float(v[(int64_t)(row0 + j) * ldv + (int64_t)h * V + c]);
+      if (MODE == 0) x = silu_f(x);
+    }
     vt[c * LK + j] = float_to_bf16_bits(x);
   }
   __syncthreads();
@@ -119,13 +147,14 @@ __global__ __launch_bounds__(256) void lightning_state_mfma_kernel(
 }
 
 // ---- pass 2: outputs of each chunk from its start state
-template <int D, int V>
+template <int D, int V, int MODE>
 __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
     float* __restrict__ out,         // [T, H, V] fp32
     const float* __restrict__ part,  // [chunks, H, V, D] start states^T
     const bf16* __restrict__ q, const bf16* __restrict__ k,
     const bf16* __restrict__ v, int64_t ldq, int64_t ldk, int64_t ldv,
-    const float* __restrict__ decay, const int* __restrict__ cu, int H) {
+    const float* __restrict__ decay, const int* __restrict__ cu, int H,
+    LmRot rot) {
   constexpr int LD = D + LM_PAD;
   constexpr int LK = LM_ROWS + LM_PAD;
   extern __shared__ __attribute__((aligned(16))) unsigned char lm_smem[];
@@ -142,8 +171,10 @@ __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
     const int j = i / D, d = i - j * D;
     float xq = 0.f, xk = 0.f;
     if (j < n) {
-      xq = silu_f(bf16_bits_to_float(q[(int64_t)(row0 + j) * ldq + (int64_t)h * D + d]));
-      xk = silu_f(bf16_bits_to_float(k[(int64_t)(row0 + j) * ldk + (int64_t)h * D + d]));
+      xq = lm_load<MODE>(q + (int64_t)(row0 + j) * ldq + (int64_t)h * D, d,
+                         row0 + j, rot);
+      xk = lm_load<MODE>(k + (int64_t)(row0 + j) * ldk + (int64_t)h * D, d,
+                         row0 + j, rot) * (MODE == 0 ? 1.f : rot.k_scale);
     }
     qs[j * LD + d] = float_to_bf16_bits(xq);
     ks[j * LD + d] = float_to_bf16_bits(xk);
@@ -151,8 +182,10 @@ __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
   for (int i = tid; i < LM_ROWS * V; i += 256) {
     const int j = i / V, c = i - j * V;
     float x = 0.f;
-    if (j < n)
-      x = silu_f(bf16_bits_to_float(v[(int64_t)(row0 + j) * ldv + (int64_t)h * V + c]));
+    if (j < n) {
+      x = bf16_bits_to_float(v[(int64_t)(row0 + j) * ldv + (int64_t)h * V + c]);
+      if (MODE == 0) x = silu_f(x);
+    }
     vt[c * LK + j] = float_to_bf16_bits(x);
   }
   const float* sp = part + ((int64_t)ch * H + h) * D * V;  // [V][D]
@@ -231,11 +264,11 @@ __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
 
 using namespace arks;
 
-template <int D, int V>
+template <int D, int V, int MODE>
 static void launch_lm(float* out, float* part, const void* q, const void* k,
                       const void* v, int64_t ldq, int64_t ldk, int64_t ldv,
                       const float* decay, const int* cu, int chunks, int H,
-                      int pass, hipStream_t stream) {
+                      int pass, LmRot rot, hipStream_t stream) {
   constexpr int LD = D + LM_PAD, LK = LM_ROWS + LM_PAD;
   dim3 grid(chunks, H), block(256);
   if (pass == 1) {
@@ -243,25 +276,25 @@ static void launch_lm(float* out, float* part, const void* q, const void* k,
     static bool set = false;
     if (!set) {
       (void)hipFuncSetAttribute(
-          reinterpret_cast<const void*>(lightning_state_mfma_kernel<D, V>),
+          reinterpret_cast<const void*>(lightning_state_mfma_kernel<D, V, MODE>),
           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
       set = true;
     }
-    hipLaunchKernelGGL((lightning_state_mfma_kernel<D, V>), grid, block, lds,
+    hipLaunchKernelGGL((lightning_state_mfma_kernel<D, V, MODE>), grid, block, lds,
                        stream, part, (const bf16*)k, (const bf16*)v, ldk, ldv,
-                       decay, cu, H);
+                       decay, cu, H, rot);
   } else {
     constexpr int lds = (2 * LM_ROWS * LD + V * LK + 2 * LM_ROWS * LK) * 2;
     static bool set = false;
     if (!set) {
       (void)hipFuncSetAttribute(
-          reinterpret_cast<const void*>(lightning_out_mfma_kernel<D, V>),
+          reinterpret_cast<const void*>(lightning_out_mfma_kernel<D, V, MODE>),
           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
       set = true;
     }
-    hipLaunchKernelGGL((lightning_out_mfma_kernel<D, V>), grid, block, lds,
+    hipLaunchKernelGGL((lightning_out_mfma_kernel<D, V, MODE>), grid, block, lds,
                        stream, out, part, (const bf16*)q, (const bf16*)k,
-                       (const bf16*)v, ldq, ldk, ldv, decay, cu, H);
+                       (const bf16*)v, ldq, ldk, ldv, decay, cu, H, rot);
   }
 }
 
@@ -272,20 +305,32 @@ extern "C" int arks_seq_lightning_mfma(void* out, void* part, const void* q,
                                        int64_t ldq, int64_t ldk, int64_t ldv,
                                        const void* decay, const void* cu,
                                        int chunks, int H, int D, int V,
-                                       int pass, hipStream_t stream) {
+                                       int pass, int mode,
+                                       const void* positions, const void* freq,
+                                       int n_rot, int interleaved,
+                                       float k_scale, hipStream_t stream) {
   if (chunks == 0) return 0;
-#define LM(DD, VV)                                                          \
-  if (D == DD && V == VV) {                                                 \
-    launch_lm<DD, VV>((float*)out, (float*)part, q, k, v, ldq, ldk, ldv,    \
-                      (const float*)decay, (const int*)cu, chunks, H, pass, \
-                      stream);                                              \
-    return 0;                                                               \
+  const LmRot rot{(const int64_t*)positions, (const float*)freq, n_rot,
+                  interleaved, k_scale};
+#define LM(DD, VV)                                                            \
+  if (D == DD && V == VV) {                                                   \
+    if (mode == 0)                                                            \
+      launch_lm<DD, VV, 0>((float*)out, (float*)part, q, k, v, ldq, ldk, ldv, \
+                           (const float*)decay, (const int*)cu, chunks, H,    \
+                           pass, rot, stream);                                \
+    else                                                                      \
+      launch_lm<DD, VV, 1>((float*)out, (float*)part, q, k, v, ldq, ldk, ldv, \
+                           (const float*)decay, (const int*)cu, chunks, H,    \
+                           pass, rot, stream);                                \
+    return 0;                                                                 \
   }
   LM(32, 32)
   LM(64, 64)
   LM(128, 128)
   LM(64, 128)
   LM(128, 64)
+  LM(64, 32)
+  LM(128, 32)
 #undef LM
   return 1;
 }

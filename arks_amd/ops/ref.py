@@ -551,3 +551,217 @@ def selective_scan(u, dbc, z, dt_w, dt_b, A, Dp, state, cu_seqlens,
 
 def gelu_tanh(x):
     return torch.nn.functional.gelu(x.float(), approximate="tanh").to(x.dtype)
+
+
+# ----------------------------------------------------------------------
+# Stream-residual blocks (several weighted copies of the residual), layer
+# norm, the short input convolution, window attention with pooled blocks,
+# rotary retention, clamped GLU and grouped routing.
+# ----------------------------------------------------------------------
+def stream_mix_norm(xs, y, y_bias, mix, out_w, in_w, norm_w, norm_b, eps):
+    """xs [s, T, C] fp32, updated in place when y is given:
+        new[t] = sum_s mix[s, t] old[s] + out_w[t] * (y + y_bias)
+    then u = sum_s in_w[s] new[s] and the layer norm of u (mean taken off,
+    variance = mean squared deviation, eps inside the root) times norm_w
+    plus norm_b -> fp32 [T, C]. in_w None: only the update."""
+    if y is not None:
+        yf = y.float()
+        if y_bias is not None:
+            yf = yf + y_bias.float()
+        new = torch.einsum("st,snc->tnc", mix.float(), xs) \
+            + out_w.float()[:, None, None] * yf[None]
+        xs.copy_(new)
+    if in_w is None:
+        return None
+    u = torch.einsum("s,snc->nc", in_w.float(), xs)
+    mu = u.mean(-1, keepdim=True)
+    d = u - mu
+    var = d.pow(2).mean(-1, keepdim=True)
+    return d * torch.rsqrt(var + eps) * norm_w.float() + norm_b.float()
+
+
+def short_conv_residual(h, weight, state, cu_seqlens, seq_lens, state_slots,
+                        out_dtype):
+    """out_t = h_t + sum_j weight[:, j] h_(t - taps + 1 + j) per channel,
+    causal within each sequence; h [T, C] fp32, weight [C, taps] fp32, state
+    [slots, taps-1, C] fp32 = each sequence's last taps-1 inputs (updated).
+    taps == 1 needs no state (state None)."""
+    T, C = h.shape
+    taps = weight.shape[1]
+    wf = weight.float()
+    out = torch.empty(T, C, dtype=torch.float32)
+    for a, b, start, slot in _seq_spans(cu_seqlens, seq_lens, state_slots):
+        hist = (state[slot].clone() if start > 0 and slot >= 0 and taps > 1
+                else torch.zeros(taps - 1, C))
+        full = torch.cat([hist, h[a:b].float()], 0)
+        n = b - a
+        acc = h[a:b].float().clone()
+        for j in range(taps):
+            acc += full[j:j + n] * wf[:, j][None, :]
+        out[a:b] = acc
+        if slot >= 0 and taps > 1:
+            state[slot] = full[n:]
+    return out.to(out_dtype)
+
+
+def pool_slots_per_page(block_size: int, pool: int) -> int:
+    """Pooled entries a page of block_size tokens can start."""
+    return (block_size - 1) // pool + 1
+
+
+def kv_write_pooled(k, v, k_cache, v_cache, kp_cache, vp_cache, slot_mapping,
+                    positions, block_tables, token_seq, pool):
+    """k [T,G,D], v [T,G,V] go to their pages; then every row whose position
+    p ends a block of `pool` positions ((p + 1) % pool == 0) leaves the mean
+    of that block's keys and values, read back from the pages (fp32 mean of
+    what the cache holds), in the pooled caches kp/vp [pages, G, spp, D|V]:
+    block b sits in the page of its first position p0 = b * pool, entry
+    (p0 % block_size) // pool."""
+    bs = k_cache.shape[2]
+    ok = slot_mapping >= 0
+    blk = (slot_mapping[ok] // bs).long()
+    off = (slot_mapping[ok] % bs).long()
+    k_cache[blk, :, off] = k[ok].to(k_cache.dtype)
+    v_cache[blk, :, off] = v[ok].to(v_cache.dtype)
+    pos = positions.tolist()
+    seqs = token_seq.tolist()
+    okl = ok.tolist()
+    for t, p in enumerate(pos):
+        if not okl[t] or (p + 1) % pool:
+            continue
+        bt = block_tables[seqs[t]]
+        p0 = p + 1 - pool
+        idx = torch.arange(p0, p + 1)
+        pages = bt[(idx // bs).long()].long()
+        offs = (idx % bs).long()
+        km = k_cache[pages, :, offs].float().mean(0)  # [G, D]
+        vm = v_cache[pages, :, offs].float().mean(0)
+        page = int(bt[p0 // bs])
+        e = (p0 % bs) // pool
+        kp_cache[page, :, e] = km.to(kp_cache.dtype)
+        vp_cache[page, :, e] = vm.to(vp_cache.dtype)
+
+
+def attention_window_pool(q, k_cache, v_cache, kp_cache, vp_cache,
+                          block_tables, seq_lens, cu_seqlens, scale, window,
+                          pool, out=None, out_scale=1.0):
+    """Softmax attention of packed new rows: the row at position i sees the
+    keys j with 0 <= i - j < window and, in the same softmax, the pooled
+    entry of every block b with b * pool + pool - 1 <= i - window.
+    q [T,H,D] -> out [T,H,V] (q.dtype), times out_scale."""
+    T, H, D = q.shape
+    G, bs, V = v_cache.shape[1], v_cache.shape[2], v_cache.shape[3]
+    res = torch.zeros(T, H, V, dtype=torch.float32)
+    cu = cu_seqlens.tolist()
+    sl = seq_lens.tolist()
+    rep = H // G
+    for s in range(len(sl)):
+        a, b = cu[s], cu[s + 1]
+        n, L = b - a, sl[s]
+        if n == 0:
+            continue
+        nbk = (L + bs - 1) // bs
+        pages = block_tables[s, :nbk].long()
+        K = k_cache[pages].permute(1, 0, 2, 3).reshape(G, nbk * bs, D)[:, :L].float()
+        Vv = v_cache[pages].permute(1, 0, 2, 3).reshape(G, nbk * bs, V)[:, :L].float()
+        nblk_max = max(0, (L - 1 - window + 1) // pool)
+        if nblk_max:
+            p0 = torch.arange(nblk_max) * pool
+            pp = block_tables[s][(p0 // bs).long()].long()
+            pe = ((p0 % bs) // pool).long()
+            KP = kp_cache[pp, :, pe].float().permute(1, 0, 2)  # [G, nb, D]
+            VP = vp_cache[pp, :, pe].float().permute(1, 0, 2)
+        for r in range(n):
+            i = L - n + r
+            lo = max(0, i - window + 1)
+            nb = (i - window + 1) // pool if i - window + 1 > 0 else 0
+            kk = K[:, lo:i + 1]
+            vv = Vv[:, lo:i + 1]
+            if nb:
+                kk = torch.cat([KP[:, :nb], kk], 1)
+                vv = torch.cat([VP[:, :nb], vv], 1)
+            kk = kk.repeat_interleave(rep, 0)  # [H, m, D]
+            vv = vv.repeat_interleave(rep, 0)
+            sc = torch.einsum("hmd,hd->hm", kk, q[a + r].float()) * scale
+            p = torch.softmax(sc, -1)
+            res[a + r] = torch.einsum("hm,hmv->hv", p, vv)
+    res = res * out_scale
+    if out is not None:
+        out.copy_(res.to(out.dtype))
+        return out
+    return res.to(q.dtype)
+
+
+def retention_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
+                   positions, inv_freq, interleaved, k_scale):
+    """Linear attention with a fixed decay per head on plain (not
+    activated) rows: q and k are turned by their position over their first
+    2*len(inv_freq) dims, k is then multiplied by k_scale;
+    S <- decay*S + k v^T, o = S^T q. -> o fp32 [T,H,V]; state updated."""
+    T, H, D = q.shape
+    V = v.shape[-1]
+    qf, kf, vf = q.float(), k.float(), v.float()
+    if inv_freq is not None and inv_freq.numel():
+        rd = 2 * inv_freq.numel()
+        ang = positions.float()[:, None, None] * inv_freq.float()[None, None, :]
+        qf = torch.cat([_rotate_pairs(qf[..., :rd], ang, interleaved), qf[..., rd:]], -1)
+        kf = torch.cat([_rotate_pairs(kf[..., :rd], ang, interleaved), kf[..., rd:]], -1)
+    kf = kf * k_scale
+    out = torch.zeros(T, H, V, dtype=torch.float32)
+    lam = decay.float()[:, None, None]
+    for a, b, start, slot in _seq_spans(cu_seqlens, seq_lens, state_slots):
+        S = (state[slot].clone() if start > 0 and slot >= 0
+             else torch.zeros(H, D, V))
+        for t in range(a, b):
+            S = lam * S + kf[t][:, :, None] * vf[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        if slot >= 0:
+            state[slot] = S
+    return out
+
+
+def head_norm_gate(o, gate, eps, heads, out, out_scale=1.0):
+    """Each head's slice of o [T, heads*V] (fp32) divided by its root mean
+    square (eps inside the root, no weight), times silu(gate), times
+    out_scale, into out [T, heads*V] (may be a column slice)."""
+    T = o.shape[0]
+    of = o.float().view(T, heads, -1)
+    y = of * torch.rsqrt(of.pow(2).mean(-1, keepdim=True) + eps)
+    g = gate.float()
+    out.copy_((y.reshape(T, -1) * g * torch.sigmoid(g) * out_scale).to(out.dtype))
+    return out
+
+
+def glu_act(gu, kind, limit=0.0, alpha=1.0):
+    """gu [T, 2F] = [gate | up] -> [T, F].
+    "swiglu": silu(gate) * up.
+    "clamped": g = min(gate, limit), u = clamp(up, -limit, limit),
+               g * sigmoid(alpha g) * (u + 1)."""
+    F_ = gu.shape[-1] // 2
+    g, u = gu[..., :F_].float(), gu[..., F_:].float()
+    if kind == "swiglu":
+        return (g * torch.sigmoid(g) * u).to(gu.dtype)
+    g = g.clamp(max=limit)
+    u = u.clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def moe_route_grouped(logits, top, groups, keep):
+    """Softmax over all experts; experts form `groups` equal runs of
+    neighbours, a group scores its best expert, only experts of the `keep`
+    best groups can be chosen; the `top` largest scores among those, their
+    scores divided by their sum (+1e-20). Ties go to the lower index.
+    logits [T, E] fp32 -> (weights [T, top] fp32, ids [T, top] int32)."""
+    s = torch.softmax(logits.float(), -1)
+    T, E = s.shape
+    per = E // groups
+    gs = s.view(T, groups, per).amax(-1)
+    kept = torch.topk(gs, keep, dim=-1).indices  # [T, keep]
+    allow = torch.zeros(T, groups, dtype=torch.bool)
+    allow.scatter_(1, kept, True)
+    masked = torch.where(allow[:, :, None].expand(T, groups, per).reshape(T, E),
+                         s, torch.full_like(s, -1.0))
+    ids = torch.topk(masked, top, dim=-1).indices
+    w = s.gather(1, ids)
+    w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    return w, ids.to(torch.int32)

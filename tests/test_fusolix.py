@@ -1,0 +1,634 @@
+"""Fusolix through the engine, and its mechanisms one by one, against the
+plain float64 model of tests/fusolix_oracle.py.
+
+Engine cases write a small random checkpoint, build an engine on it and
+replay a step plan with the product's trace replay (the scheduler's pages
+and state slots, the runner's batches, the model's kernels); op cases drive
+single ops with inputs made so that a fault shows (one key that must win,
+keys on both sides of a window's or a pooled block's edge). CPU cases run
+the reference ops, gpu-marked ones the HIP kernels in float32 and bfloat16.
+"""
+
+import io
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import fusolix_oracle as O
+
+CASES = [
+    pytest.param("cpu", "float32", id="cpu-f32"),
+    pytest.param("cuda", "float32", id="gpu-f32", marks=pytest.mark.gpu),
+    pytest.param("cuda", "bfloat16", id="gpu-bf16", marks=pytest.mark.gpu),
+]
+TOL = {"float32": 2e-4, "bfloat16": 6e-2}
+TDT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+F64 = torch.float64
+
+
+# ------------------------------------------------------------------ helpers
+def write_checkpoint(path, cfg, seed=0):
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    w = O.random_weights(cfg, seed)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in w.items()},
+              os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return w
+
+
+def make_engine(path, device, dtype, max_tokens=256, **kw):
+    from arks_amd.config import EngineConfig
+    from arks_amd.engine import LLMEngine
+
+    cfg = EngineConfig(model_path=str(path), device=device, dtype=dtype,
+                       kv_cache_blocks=-(-max_tokens // 16), max_num_seqs=4,
+                       max_model_len=max_tokens, max_num_batched_tokens=max_tokens,
+                       enable_prefix_caching=False, **kw)
+    return LLMEngine(cfg)
+
+
+def replay(engine, tmp_path, steps):
+    """steps: lists of (request id, tokens, end?); logits of every token.
+    Returns {id: [n_tokens, vocab]}."""
+    from arks_amd.engine.trace import replay as trace_replay
+
+    out = tmp_path / "out"
+    out.mkdir(exist_ok=True)
+    lines = [json.dumps({
+        "step": n,
+        "entries": [{"id": i, "tokens": t, "want": list(range(len(t)))}
+                    for i, t, _ in step],
+        "end": [i for i, _, e in step if e]}) for n, step in enumerate(steps)]
+    trace_replay(engine, lines, str(out), log=io.StringIO())
+    got = {}
+    V = engine.model_cfg.vocab_size
+    for n, step in enumerate(steps):
+        arr = np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, V)
+        at = 0
+        for i, t, _ in step:
+            got.setdefault(i, []).append(arr[at:at + len(t)])
+            at += len(t)
+    return {i: np.concatenate(v) for i, v in got.items()}
+
+
+def rel_err(got, want):
+    want = want.numpy() if isinstance(want, torch.Tensor) else want
+    d = got - want
+    return float(np.sqrt((d ** 2).mean(-1)).max() / np.sqrt((want ** 2).mean()))
+
+
+def portions(tokens, sizes):
+    out, at, k = [], 0, 0
+    while at < len(tokens):
+        n = sizes[k % len(sizes)]
+        out.append(tokens[at:at + n])
+        at += n
+        k += 1
+    return out
+
+
+def toks(n, vocab=96, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def oracle_logits(cfg, w, t):
+    return O.forward(cfg, w, t)[0]
+
+
+# --------------------------------------------------- the model in the engine
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("layers", [(None,), ("dense",), ("moe",)],
+                         ids=["mixer", "mixer+dense", "mixer+moe"])
+def test_one_layer(tmp_path, device, dtype, layers):
+    cfg = O.make_config(layers=layers)
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(45)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    got = replay(eng, tmp_path, [[("a", t, True)]])["a"]
+    assert rel_err(got, oracle_logits(cfg, w, t)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_residual_after_every_layer(tmp_path, device, dtype):
+    cfg = O.make_config(layers=("dense", None, "moe"))
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(21)
+    _, sums = O.forward(cfg, w, t)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    seen = {}
+    eng.runner.model.residual_tap = lambda i, x: seen.__setitem__(i, x.float().cpu())
+    replay(eng, tmp_path, [[("a", t, True)]])
+    for i, want in enumerate(sums):
+        assert rel_err(seen[i].numpy(), want) < TOL[dtype], i
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_prefill_against_decode_and_portions(tmp_path, device, dtype):
+    """One prompt whole, token by token, and in portions down to two
+    tokens: window 8 and pool 4 are crossed many times in each."""
+    cfg = O.make_config()
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(70)
+    want = oracle_logits(cfg, w, t)
+    for name, plan in {
+        "decode": [t[:9]] + [[x] for x in t[9:]],
+        "small": portions(t, [2, 3, 5, 2, 7]),
+        "odd": portions(t, [13, 1, 2, 17]),
+        "tokens": [[x] for x in t[:40]],
+    }.items():
+        eng = make_engine(tmp_path / "m", device, dtype)
+        steps = [[("a", p, False)] for p in plan]
+        got = replay(eng, tmp_path, steps)["a"]
+        assert rel_err(got, want[:len(got)]) < TOL[dtype], name
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_mixed_batches_and_reuse(tmp_path, device, dtype):
+    """Unequal requests side by side, portions beside single tokens; more
+    requests than state slots over time and a pool just large enough, so
+    pages and slots are given back and taken again."""
+    cfg = O.make_config(layers=("moe", "dense"))
+    w = write_checkpoint(tmp_path / "m", cfg)
+    reqs = {c: toks(n, seed=s) for c, n, s in
+            [("a", 61, 1), ("b", 18, 2), ("c", 33, 3), ("d", 5, 4),
+             ("e", 47, 5), ("f", 29, 6), ("g", 40, 7)]}
+    want = {c: oracle_logits(cfg, w, t) for c, t in reqs.items()}
+    at = {c: 0 for c in reqs}
+    order = list(reqs)
+    live, waiting, steps = [], order[:], []
+    sizes = [7, 1, 2, 16, 1, 1, 3, 11]
+    k = 0
+    while live or waiting:
+        while waiting and len(live) < 4 and \
+                sum(-(-len(reqs[c]) // 16) for c in live + waiting[:1]) <= 12:
+            live.append(waiting.pop(0))
+        step = []
+        for c in list(live):
+            if (k + ord(c)) % 5 == 0 and len(live) > 1:
+                k += 1
+                continue  # this request sits the step out
+            n = min(sizes[k % len(sizes)], len(reqs[c]) - at[c])
+            k += 1
+            part = reqs[c][at[c]:at[c] + n]
+            at[c] += n
+            done = at[c] == len(reqs[c])
+            step.append((c, part, done))
+            if done:
+                live.remove(c)
+        if step:
+            steps.append(step)
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=192)
+    got = replay(eng, tmp_path, steps)
+    for c in reqs:
+        assert got[c].shape[0] == len(reqs[c])
+        assert rel_err(got[c], want[c]) < TOL[dtype], c
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_long_decode(tmp_path, device, dtype):
+    cfg = O.make_config(layers=("dense",), window=24, pool=16)
+    w = write_checkpoint(tmp_path / "m", cfg)
+    t = toks(150)
+    want = oracle_logits(cfg, w, t)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    steps = [[("a", t[:5], False)]] + [[("a", [x], False)] for x in t[5:]]
+    got = replay(eng, tmp_path, steps)["a"]
+    assert rel_err(got, want) < TOL[dtype]
+
+
+OTHER_SIZES = {
+    "one-stream-no-conv-history": dict(streams=1, taps=1, layers=("dense",)),
+    "three-streams-five-taps": dict(streams=3, taps=5, layers=("moe", None)),
+    "pool-above-page": dict(pool=24, window=7, layers=("dense",)),
+    "pool-not-dividing-page": dict(pool=5, window=3, layers=(None,)),
+    "pool-one-window-one": dict(pool=1, window=1, layers=(None,)),
+    "window-above-prompt": dict(window=500, pool=8, layers=("dense",)),
+    "all-kv-heads": dict(heads=3, kv_heads=3, dim=8, vdim=24, layers=(None,)),
+    "one-kv-head-odd-dims": dict(heads=6, kv_heads=1, dim=24, vdim=8,
+                                 r_heads=3, r_dim=12, r_vdim=20, rot_dims=4,
+                                 decay=(0.5, 0.999, 1.0), width=40,
+                                 layers=("dense",)),
+    "full-rotary-no-rotary": dict(rot_dims=16, layers=(None,)),
+    "no-rotary": dict(rot_dims=0, layers=(None,)),
+    "every-group-kept-top-one": dict(experts=8, groups=4, keep=4, top=1,
+                                     layers=("moe",)),
+    "one-group": dict(experts=5, groups=1, keep=1, top=3, layers=("moe",)),
+    "one-expert-per-group": dict(experts=6, groups=6, keep=2, top=2,
+                                 layers=("moe",)),
+    "scales": dict(left_scale=0.0, right_scale=2.5, embed_scale=1.0,
+                   limit=0.25, layers=("dense",)),
+}
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("name", list(OTHER_SIZES))
+def test_other_sizes(tmp_path, device, dtype, name):
+    cfg = O.make_config(**OTHER_SIZES[name])
+    w = write_checkpoint(tmp_path / "m", cfg, seed=3)
+    t = toks(58, vocab=cfg["vocab"])
+    want = oracle_logits(cfg, w, t)
+    eng = make_engine(tmp_path / "m", device, dtype)
+    steps = [[("a", p, False)] for p in portions(t[:37], [9, 2, 1, 6])] + \
+            [[("a", [x], False)] for x in t[37:]]
+    got = replay(eng, tmp_path, steps)["a"]
+    assert rel_err(got, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("device,dtype", [
+    pytest.param("cuda", "float32", id="gpu-f32", marks=pytest.mark.gpu),
+    pytest.param("cuda", "bfloat16", id="gpu-bf16", marks=pytest.mark.gpu)])
+def test_matrix_core_sizes(tmp_path, device, dtype):
+    """Head sizes the matrix-core kernels are built for, prompts long
+    enough for their chunked paths, portions across 64-row edges."""
+    cfg = O.make_config(width=128, heads=4, kv_heads=2, dim=64, vdim=64,
+                        r_heads=2, r_dim=64, r_vdim=32, rot_dims=32,
+                        window=40, pool=8, layers=("dense", "moe"))
+    w = write_checkpoint(tmp_path / "m", cfg)
+    reqs = {"a": toks(300, seed=1), "b": toks(131, seed=2)}
+    want = {c: oracle_logits(cfg, w, t) for c, t in reqs.items()}
+    eng = make_engine(tmp_path / "m", device, dtype, max_tokens=512)
+    a, b = reqs["a"], reqs["b"]
+    steps = [[("a", a[:130], False), ("b", b[:3], False)],
+             [("a", a[130:199], False), ("b", b[3:4], False)],
+             [("a", a[199:], True), ("b", b[4:], True)]]
+    got = replay(eng, tmp_path, steps)
+    for c in reqs:
+        assert rel_err(got[c], want[c]) < TOL[dtype], c
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_greedy_generation(tmp_path, device, dtype):
+    """LLMEngine.generate (scheduler, sampler, captured decode steps on the
+    GPU) picks the oracle's tokens; three prompts share the batch."""
+    from arks_amd.engine import SamplingParams
+
+    cfg = O.make_config(layers=("dense", "moe"))
+    w = write_checkpoint(tmp_path / "m", cfg)
+    prompts = [toks(19, seed=4), toks(3, seed=5), toks(34, seed=6)]
+    eng = make_engine(tmp_path / "m", device, dtype)
+    outs = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True,
+                                                temperature=0.0))
+    for p, o in zip(prompts, outs):
+        seq = list(p)
+        for tok in o:
+            logits = oracle_logits(cfg, w, seq)[-1]
+            top2 = torch.topk(logits, 2).values
+            if float(top2[0] - top2[1]) > (1e-3 if dtype == "float32" else 0.15):
+                assert tok == int(logits.argmax()), (len(seq), tok)
+            seq.append(tok)
+
+
+# ------------------------------------------------------- mechanisms alone
+def _dev(device):
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return torch.device(device)
+
+
+def _meta(lens_new, lens_total, dev):
+    cu = [0]
+    for n in lens_new:
+        cu.append(cu[-1] + n)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    token_seq = [s for s, n in enumerate(lens_new) for _ in range(n)]
+    return i32(cu), i32(lens_total), i32(token_seq)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("streams", [1, 2, 4])
+def test_stream_mix_norm(device, dtype, streams):
+    from arks_amd import ops
+
+    dev = _dev(device)
+    g = torch.Generator().manual_seed(streams)
+    T, C = 7, 52
+    xs = torch.randn(streams, T, C, generator=g, dtype=F64)
+    y = torch.randn(T, C, generator=g, dtype=F64).to(TDT[dtype]).to(F64)
+    bias = torch.randn(C, generator=g, dtype=F64)
+    mix = torch.randn(streams, streams, generator=g, dtype=F64)
+    ow, iw = (torch.randn(streams, generator=g, dtype=F64) for _ in range(2))
+    nw, nb = (torch.randn(C, generator=g, dtype=F64) for _ in range(2))
+    new = O.streams_write(xs, y + bias, mix, ow)
+    want = O.layer_norm(O.streams_read(new, iw), nw, nb, 1e-5)
+    f = lambda t: t.float().to(dev)
+    xd = f(xs).contiguous()
+    n = ops.stream_mix_norm(xd, y.to(TDT[dtype]).to(dev), f(bias), f(mix), f(ow),
+                            f(iw), f(nw), f(nb), 1e-5)
+    assert torch.allclose(xd.cpu().double(), new, atol=1e-4, rtol=1e-5)
+    assert torch.allclose(n.cpu().double(), want, atol=2e-4, rtol=1e-4)
+    # update only, then read only
+    xd2 = f(xs).contiguous()
+    assert ops.stream_mix_norm(xd2, y.to(TDT[dtype]).to(dev), None, f(mix), f(ow),
+                               None, None, None, 1e-5) is None
+    new2 = O.streams_write(xs, y, mix, ow)
+    assert torch.allclose(xd2.cpu().double(), new2, atol=1e-4, rtol=1e-5)
+    n2 = ops.stream_mix_norm(xd2, None, None, None, None, f(iw), f(nw), f(nb), 1e-5)
+    want2 = O.layer_norm(O.streams_read(new2, iw), nw, nb, 1e-5)
+    assert torch.allclose(n2.cpu().double(), want2, atol=2e-4, rtol=1e-4)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("taps", [1, 2, 4, 6])
+def test_short_conv_portions(device, dtype, taps):
+    """Two sequences in portions of 1, 2 and more rows sharing steps; the
+    history crosses every portion edge; slots hold another sequence's
+    leftovers first."""
+    from arks_amd import ops
+
+    dev = _dev(device)
+    g = torch.Generator().manual_seed(taps)
+    C = 40
+    w = torch.randn(C, taps, generator=g, dtype=F64)
+    seqs = [torch.randn(n, C, generator=g, dtype=F64) for n in (23, 9)]
+    want = [O.short_conv_residual(h, w) for h in seqs]
+    state = (torch.full((3, taps - 1, C), 7.0, device=dev) if taps > 1 else None)
+    slots = torch.tensor([2, 0], dtype=torch.int32, device=dev)
+    plans = [portions(list(range(23)), [1, 2, 5, 1, 1, 3]),
+             portions(list(range(9)), [2, 1, 1])]
+    at = [0, 0]
+    got = [[], []]
+    for step in range(max(len(p) for p in plans)):
+        new = [len(p[step]) if step < len(p) else 0 for p in plans]
+        rows = torch.cat([seqs[s][at[s]:at[s] + new[s]] for s in range(2)])
+        cu, lens, ts = _meta(new, [at[s] + new[s] for s in range(2)], dev)
+        out = ops.short_conv_residual(rows.float().to(dev), w.float().to(dev),
+                                      state, cu, lens, slots, ts, TDT[dtype])
+        o = out.cpu().double()
+        for s in range(2):
+            got[s].append(o[int(cu[s]):int(cu[s + 1])])
+            at[s] += new[s]
+    tol = 1e-4 if dtype == "float32" else 5e-2
+    for s in range(2):
+        assert torch.allclose(torch.cat(got[s]), want[s], atol=tol, rtol=tol)
+
+
+class PagedWindow:
+    """Keys/values of one sequence written into shuffled pages, in steps."""
+
+    def __init__(self, dev, dtype, G, D, V, pool, total, seed=0, bs=16):
+        from arks_amd import ops
+
+        self.ops, self.dev, self.dt = ops, dev, TDT[dtype]
+        self.G, self.D, self.V, self.pool, self.bs = G, D, V, pool, bs
+        nblk = -(-total // bs)
+        g = torch.Generator().manual_seed(seed)
+        npages = nblk + 5
+        self.table = torch.randperm(npages, generator=g)[:nblk].to(torch.int32)
+        spp = ops.pool_slots_per_page(bs, pool)
+        z = lambda *s: torch.full(s, 3.0, dtype=self.dt, device=dev)  # junk
+        self.kc, self.vc = z(npages, G, bs, D), z(npages, G, bs, V)
+        self.kp, self.vp = z(npages, G, spp, D), z(npages, G, spp, V)
+        self.bt = self.table[None].to(dev)
+        self.at = 0
+
+    def step(self, q, k, v, scale, window, out_scale=1.0):
+        """q [n,H,D], k [n,G,D], v [n,G,V] (float64) -> out [n,H,V]."""
+        n = q.shape[0]
+        pos = torch.arange(self.at, self.at + n)
+        slot = (self.table[(pos // self.bs).long()].long() * self.bs
+                + pos % self.bs).to(self.dev)
+        cu, lens, ts = _meta([n], [self.at + n], self.dev)
+        c = lambda t: t.to(self.dt).to(self.dev)
+        self.ops.kv_write_pooled(c(k), c(v), self.kc, self.vc, self.kp, self.vp,
+                                 slot, pos.to(self.dev), self.bt, ts, self.pool)
+        out = torch.empty(n, q.shape[1], self.V, dtype=self.dt, device=self.dev)
+        self.ops.attention_window_pool(
+            c(q), self.kc, self.vc, self.kp, self.vp, self.bt, lens, cu, ts,
+            scale, window, self.pool, out, out_scale, n)
+        self.at += n
+        return out.float().cpu().double()
+
+
+def _rounded(t, dtype):
+    return t.to(TDT[dtype]).to(F64)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("window,pool,plan", [
+    (8, 4, [37, 1, 1, 2, 30]), (96, 16, [130, 1, 70, 1]), (5, 24, [3, 50, 1, 1, 64]),
+    (16, 5, [1] * 45), (1, 1, [20, 1, 9]), (33, 16, [200]),
+], ids=["w8p4", "w96p16", "w5p24", "w16p5-decode", "w1p1", "w33p16-whole"])
+def test_window_pool_attention(device, dtype, window, pool, plan):
+    dev = _dev(device)
+    H, G, D, V = 4, 2, 16, 16
+    n = sum(plan)
+    g = torch.Generator().manual_seed(window * 100 + pool)
+    q = _rounded(torch.randn(n, H, D, generator=g, dtype=F64), dtype)
+    k = _rounded(torch.randn(n, G, D, generator=g, dtype=F64), dtype)
+    v = _rounded(torch.randn(n, G, V, generator=g, dtype=F64), dtype)
+    want = O.window_pool_attention(q, k, v, 0.4, window, pool) * 0.7
+    pw = PagedWindow(dev, dtype, G, D, V, pool, n)
+    got, at = [], 0
+    for m in plan:
+        got.append(pw.step(q[at:at + m], k[at:at + m], v[at:at + m], 0.4,
+                           window, 0.7))
+        at += m
+    tol = 2e-4 if dtype == "float32" else 3e-2
+    assert torch.allclose(torch.cat(got), want, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("decode", [False, True], ids=["prompt", "decoded"])
+def test_window_and_pool_edges_decide(device, dtype, decode):
+    """Among hundreds of keys one gets a huge score. Where it sits decides
+    what the row returns: the last key inside the window gives its value,
+    the first key outside it (its block not yet complete behind the window)
+    is invisible, a key in a block just behind the window shows through the
+    block's mean, one block further on it is invisible again."""
+    dev = _dev(device)
+    H, G, D, V = 2, 1, 16, 16
+    window, pool, n = 20, 8, 300
+    i = n - 1                      # the row that asks
+    nb = (i - window + 1) // pool  # blocks it sees: 35 -> positions < 280
+    assert nb * pool == i - window + 1  # blocks end right at the window
+    g = torch.Generator().manual_seed(5)
+    base_k = torch.randn(n, G, D, generator=g, dtype=F64) * 0.1
+    v = _rounded(torch.randn(n, G, V, generator=g, dtype=F64), dtype)
+    e = torch.zeros(D, dtype=F64)
+    e[3] = 1.0
+    for hot, seen in [(i - window + 1, "token"), (i - window, "block"),
+                      (nb * pool - pool, "block"), (3, "block"),
+                      (i, "token")]:
+        k = base_k.clone()
+        k[hot, 0] = 40.0 * e
+        k = _rounded(k, dtype)
+        q = torch.zeros(n, H, D, dtype=F64)
+        q[i, :] = 8.0 * e
+        want = O.window_pool_attention(q, k, v, 0.5, window, pool)[i]
+        ref_val = v[hot, 0] if seen == "token" else \
+            v[hot // pool * pool:hot // pool * pool + pool, 0].mean(0)
+        assert torch.allclose(want[0], ref_val, atol=1e-6), (hot, seen)
+        pw = PagedWindow(dev, dtype, G, D, V, pool, n)
+        cut = n - 1 if decode else n - 37
+        pw.step(q[:cut], k[:cut], v[:cut], 0.5, window)
+        got = pw.step(q[cut:], k[cut:], v[cut:], 0.5, window)[-1]
+        tol = 1e-4 if dtype == "float32" else 2e-2
+        assert torch.allclose(got, want, atol=tol, rtol=tol), (hot, seen)
+    # a window that ends inside a block: the keys between the last complete
+    # block and the window are seen by nobody
+    window = 23
+    lo = i - window + 1
+    nb = lo // pool
+    assert nb * pool < lo
+    hot = lo - 1
+    k = base_k.clone()
+    k[hot, 0] = 40.0 * e
+    k = _rounded(k, dtype)
+    q = torch.zeros(n, H, D, dtype=F64)
+    q[i, :] = 8.0 * e
+    want = O.window_pool_attention(q, k, v, 0.5, window, pool)[i]
+    assert not torch.allclose(want[0], v[hot, 0], atol=0.05)
+    pw = PagedWindow(dev, dtype, G, D, V, pool, n)
+    cut = n - 1 if decode else n - 37
+    pw.step(q[:cut], k[:cut], v[:cut], 0.5, window)
+    got = pw.step(q[cut:], k[cut:], v[cut:], 0.5, window)[-1]
+    tol = 1e-4 if dtype == "float32" else 2e-2
+    assert torch.allclose(got, want, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16"])
+@pytest.mark.gpu
+@pytest.mark.parametrize("D,V", [(64, 64), (128, 128), (128, 64), (64, 128),
+                                 (32, 32), (96, 96)])
+def test_window_matrix_core_kernel_against_general(dtype, D, V):
+    from arks_amd import ops
+
+    dev = _dev("cuda")
+    H, G = 4, 2
+    window, pool = 70, 16
+    plan = [250, 3, 64, 65, 1, 130]
+    n = sum(plan)
+    g = torch.Generator().manual_seed(D + V)
+    q = _rounded(torch.randn(n, H, D, generator=g, dtype=F64), dtype)
+    k = _rounded(torch.randn(n, G, D, generator=g, dtype=F64), dtype)
+    v = _rounded(torch.randn(n, G, V, generator=g, dtype=F64), dtype)
+    outs = {}
+    for fast in (True, False):
+        ops.use_window_mfma = fast
+        try:
+            pw = PagedWindow(dev, dtype, G, D, V, pool, n)
+            got, at = [], 0
+            for m in plan:
+                got.append(pw.step(q[at:at + m], k[at:at + m], v[at:at + m],
+                                   D ** -0.5, window))
+                at += m
+            outs[fast] = torch.cat(got)
+        finally:
+            ops.use_window_mfma = True
+    assert torch.allclose(outs[True], outs[False], atol=2e-2, rtol=2e-2)
+    want = O.window_pool_attention(q, k, v, D ** -0.5, window, pool)
+    assert torch.allclose(outs[True], want, atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+@pytest.mark.parametrize("rot_dims,interleaved", [(0, False), (6, False),
+                                                  (16, False), (8, True)])
+def test_retention_scan(device, dtype, rot_dims, interleaved):
+    """Portions of 1, 2 and many rows (above the 64-row chunk on the GPU),
+    state carried in a slot that held junk; decay 1 and a fast decay."""
+    from arks_amd import ops
+    from arks_amd.models.mixers import rotary_inv_freq
+
+    dev = _dev(device)
+    H, D, V, n = 3, 16, 8, 171
+    decay = [1.0, 0.5, 0.99]
+    g = torch.Generator().manual_seed(rot_dims)
+    q, k = (_rounded(torch.randn(n, H, D, generator=g, dtype=F64), dtype)
+            for _ in range(2))
+    v = _rounded(torch.randn(n, H, V, generator=g, dtype=F64), dtype)
+    pos = torch.arange(n)
+    if interleaved:
+        # the same turn in the other pairing: permute dims, use the oracle
+        perm = torch.cat([torch.arange(0, rot_dims, 2),
+                          torch.arange(1, rot_dims, 2),
+                          torch.arange(rot_dims, D)])
+        qo = O.rotate_half_split(q[..., perm], pos, 50.0, rot_dims)
+        ko = O.rotate_half_split(k[..., perm], pos, 50.0, rot_dims)
+    elif rot_dims:
+        qo = O.rotate_half_split(q, pos, 50.0, rot_dims)
+        ko = O.rotate_half_split(k, pos, 50.0, rot_dims)
+    else:
+        qo, ko = q, k
+    want = O.retention(qo, ko * 0.3, v, decay)
+    state = torch.full((2, H, D, V), 9.0, device=dev)
+    inv = rotary_inv_freq(50.0, rot_dims).to(dev) if rot_dims else None
+    dec = torch.tensor(decay, device=dev)
+    slots = torch.tensor([1], dtype=torch.int32, device=dev)
+    got, at = [], 0
+    for m in [1, 2, 70, 1, 65, 3, 29]:
+        cu, lens, _ = _meta([m], [at + m], dev)
+        c = lambda t: t[at:at + m].to(TDT[dtype]).to(dev)
+        chunks = ops.scan_chunks([m], dev) if device == "cuda" and m > 64 else None
+        o = ops.retention_scan(c(q), c(k), c(v), dec, state, cu, lens, slots,
+                               pos[at:at + m].to(dev), inv, interleaved, 0.3,
+                               m, chunks)
+        got.append(o.cpu().double())
+        at += m
+    got = torch.cat(got)
+    scale = float(want.abs().max())
+    tol = 2e-4 if dtype == "float32" else 2e-2
+    assert float((got - want).abs().max()) < tol * scale
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
+def test_head_norm_gate_and_glu(device, dtype):
+    from arks_amd import ops
+
+    dev = _dev(device)
+    g = torch.Generator().manual_seed(0)
+    T, H, V = 5, 3, 24
+    o = torch.randn(T, H, V, generator=g, dtype=F64) * 3
+    gate = _rounded(torch.randn(T, H * V, generator=g, dtype=F64), dtype)
+    want = O.unit_rms(o, 1e-5).reshape(T, -1) * gate * torch.sigmoid(gate) * 1.5
+    wide = torch.zeros(T, H * V + 16, dtype=TDT[dtype], device=dev)
+    ops.head_norm_gate(o.reshape(T, -1).float().to(dev),
+                       gate.to(TDT[dtype]).to(dev), 1e-5, H, wide[:, 16:], 1.5)
+    tol = 1e-4 if dtype == "float32" else 3e-2
+    assert torch.allclose(wide[:, 16:].float().cpu().double(), want, atol=tol, rtol=tol)
+    assert float(wide[:, :16].abs().max()) == 0.0
+    gu = _rounded(torch.randn(T, 2 * 40, generator=g, dtype=F64) * 3, dtype)
+    a, u = gu[:, :40], gu[:, 40:]
+    lim = 1.25
+    a2 = a.clamp(max=lim)
+    want = a2 * torch.sigmoid(1.702 * a2) * (u.clamp(-lim, lim) + 1)
+    got = ops.glu_act(gu.to(TDT[dtype]).to(dev), "clamped", lim, 1.702)
+    assert torch.allclose(got.float().cpu().double(), want, atol=tol, rtol=tol)
+    want = a * torch.sigmoid(a) * u
+    got = ops.glu_act(gu.to(TDT[dtype]).to(dev), "swiglu")
+    assert torch.allclose(got.float().cpu().double(), want, atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("device", [
+    "cpu", pytest.param("cuda", marks=pytest.mark.gpu)])
+@pytest.mark.parametrize("E,groups,keep,top", [
+    (16, 2, 1, 2), (12, 4, 2, 3), (8, 8, 3, 2), (6, 1, 1, 6), (64, 8, 4, 8)])
+def test_grouped_routing(device, E, groups, keep, top):
+    """Also rows where the best experts sit in a group that loses: the
+    second-best expert overall must not be chosen when its group's best is
+    below another group's."""
+    from arks_amd import ops
+
+    dev = _dev(device)
+    g = torch.Generator().manual_seed(E)
+    z = torch.randn(40, E, generator=g) * 2
+    if groups > keep:
+        per = E // groups
+        z[0] = -3.0
+        z[0, 0] = 5.0            # best: group 0
+        z[0, per] = 4.0          # second best overall, in group 1
+        if per > 1:
+            z[0, 1] = 1.0
+    w, ids = ops.moe_route_grouped(z.to(dev), top, groups, keep)
+    for t in range(z.shape[0]):
+        wi, ww = O.route(z[t].double(), top, groups, keep)
+        assert sorted(ids[t].tolist()) == sorted(wi), t
+        got = dict(zip(ids[t].tolist(), w[t].tolist()))
+        for e, c in zip(wi, ww):
+            assert abs(got[e] - c) < 1e-5
