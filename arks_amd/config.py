@@ -256,6 +256,34 @@ def _gagorax_preset(width, vocab, pattern, heads, kv_heads, dim, ff,
                              rms_norm_eps=1e-5, logit_scale=1.0)
 
 
+def _fusolix_preset(width, vocab, pattern, heads, kv_heads, dim, window, pool,
+                    r_heads, r_dim, r_vdim, ff, experts, top, groups, keep,
+                    expert_ff, streams=2, taps=4) -> HybridModelConfig:
+    """pattern: one letter per layer for its feed-forward, d (dense), m
+    (experts) or n (none); every layer has the parallel mixer."""
+    layers = []
+    for ch in pattern:
+        mixer = {
+            "left": {"heads": heads, "kv_heads": kv_heads, "dim": dim,
+                     "vdim": dim, "scale": dim ** -0.5,
+                     "mask": {"size": window, "pool": pool}},
+            "right": {"heads": r_heads, "dim": r_dim, "vdim": r_vdim,
+                      "decay": [1.0 - 2.0 ** (-5 - 5 * h / max(r_heads - 1, 1))
+                                for h in range(r_heads)],
+                      "rot": {"base": 10000.0, "dims": r_dim // 2}},
+            "left_scale": 1.0, "right_scale": 1.0}
+        mlp = ({"kind": "dense", "ff": ff, "limit": 7.0} if ch == "d" else
+               {"kind": "moe", "expert": {"ff": expert_ff},
+                "router": {"experts": experts, "top": top,
+                           "groups": {"count": groups, "keep": keep}}}
+               if ch == "m" else None)
+        layers.append({"type": "parallel", "mixer": mixer, "mlp": mlp})
+    return HybridModelConfig(
+        architecture="Fusolix", vocab_size=vocab, hidden_size=width,
+        layers=layers, rms_norm_eps=1e-5, streams=streams, conv_taps=taps,
+        embed_scale=1.0)
+
+
 # Named synthetic configs for benchmarks / tests (random-init weights; no
 # network access for real checkpoints — BASELINE.json's models by shape).
 PRESET_CONFIGS: dict[str, ModelConfig] = {
@@ -531,6 +559,15 @@ PRESET_CONFIGS: dict[str, ModelConfig] = {
         4096, 32000, "almmalmm", 32, 8, 128, 14336, 8192, 16, 256, 32, 128),
     "tiny-gagorax": _gagorax_preset(
         128, 512, "alma", 4, 2, 32, 192, 160, 8, 12, 2, 16),
+    # Fusolix at the layer sizes of an ~8B model: 32/8 heads x 128 over a
+    # 1024-token window with 64-token pooled blocks beside 16 retention
+    # heads x 128; dense ff 14336 alternating with 16 experts of ff 3584
+    # (4 of them per row, from 2 of 4 groups)
+    "fusolix-8b-slice": _fusolix_preset(
+        4096, 32000, "dmdmdmdm", 32, 8, 128, 1024, 64, 16, 128, 128, 14336,
+        16, 4, 4, 2, 3584),
+    "tiny-fusolix": _fusolix_preset(
+        128, 512, "dmn", 4, 2, 32, 24, 8, 2, 32, 16, 192, 8, 2, 4, 2, 48),
     "tiny-gpu": ModelConfig(  # GPU-test-sized (head_dim 128 kernels)
         architecture="Qwen2ForCausalLM",
         vocab_size=2048,

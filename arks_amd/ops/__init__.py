@@ -905,11 +905,11 @@ def attention_window_pool(q, k_cache, v_cache, kp_cache, vp_cache,
     column slice of a wider row), scaled by out_scale."""
     if q.is_cuda:
         S = _native_seq()
-        if not (use_window_mfma and q.dtype == torch.bfloat16 and max_q_len > 1
+        if not (use_window_mfma and q.dtype == torch.bfloat16
                 and S.attention_window_pool_mfma(
                     out, q, k_cache, v_cache, kp_cache, vp_cache, block_tables,
                     seq_lens, cu_seqlens, token_seq, scale, window, pool,
-                    out_scale)):
+                    out_scale, max_q_len == 1)):
             S.attention_window_pool(
                 out, q, k_cache, v_cache, kp_cache, vp_cache, block_tables,
                 seq_lens, cu_seqlens, token_seq, scale, window, pool,

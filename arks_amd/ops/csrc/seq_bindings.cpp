@@ -115,7 +115,8 @@ int arks_seq_attn_window_pool_mfma(void* out, int64_t ldo, const void* q,
                                    int window, int pool, int spp,
                                    float out_scale, int T, int H, int G, int D,
                                    int V, int bs, int max_blocks,
-                                   int num_seqs, hipStream_t stream);
+                                   int num_seqs, int single_rows,
+                                   hipStream_t stream);
 int arks_seq_moe_route_grouped(void* weights, void* ids, const void* logits,
                                int T, int E, int top, int groups, int keep,
                                hipStream_t stream);
@@ -792,12 +793,14 @@ void attention_window_pool(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
 }
 
 // The matrix-core kernel; false: not built for these sizes (the caller
-// runs the general kernel).
+// runs the general kernel). single_rows: every sequence has one row in
+// this step (a workgroup then takes the query heads of one group).
 bool attention_window_pool_mfma(Tensor out, Tensor q, Tensor k_cache,
                                 Tensor v_cache, Tensor kp, Tensor vp,
                                 Tensor block_tables, Tensor seq_lens, Tensor cu,
                                 Tensor token_seq, double scale, int64_t window,
-                                int64_t pool, double out_scale) {
+                                int64_t pool, double out_scale,
+                                bool single_rows) {
   const WindowShapes w = check_window(q, k_cache, v_cache, kp, vp,
                                       block_tables, pool);
   TORCH_CHECK(w.f32 == 0, "bf16 rows only");
@@ -812,7 +815,8 @@ bool attention_window_pool_mfma(Tensor out, Tensor q, Tensor k_cache,
              seq_lens.data_ptr(), cu.data_ptr(), token_seq.data_ptr(),
              (float)scale, (int)window, (int)pool, w.spp, (float)out_scale,
              w.T, w.H, w.G, w.D, w.V, w.bs, w.max_blocks,
-             (int)seq_lens.numel(), current_stream()) == 0;
+             (int)seq_lens.numel(), single_rows ? 1 : 0,
+             current_stream()) == 0;
 }
 
 void moe_route_grouped(Tensor weights, Tensor ids, Tensor logits, int64_t top,

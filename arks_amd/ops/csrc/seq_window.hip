@@ -34,38 +34,87 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
   }
 }
 
-// One block per (row, kv head); only rows whose position ends a block work.
-// Runs after kv_write_kernel on the same stream, so it sees this step's rows.
+// One block per (64 rows, kv head): the rows whose position ends a block are
+// listed first (one in `pool` of a prompt's rows), then the block's waves
+// share them, lanes over the key and value dims. Runs after kv_write_kernel
+// on the same stream, so it sees this step's rows.
 template <typename AT>
-__global__ __launch_bounds__(64) void kv_pool_kernel(
+__global__ __launch_bounds__(256) void kv_pool_kernel(
     const AT* __restrict__ k_cache, const AT* __restrict__ v_cache,
     AT* __restrict__ kp_cache, AT* __restrict__ vp_cache,
     const int64_t* __restrict__ slot_mapping,
     const int64_t* __restrict__ positions, const int* __restrict__ block_tables,
-    const int* __restrict__ token_seq, int max_blocks, int G, int D, int V,
-    int bs, int pool, int spp) {
-  const int t = blockIdx.x, g = blockIdx.y;
-  if (slot_mapping[t] < 0) return;
-  const int64_t p = positions[t];
-  if ((p + 1) % pool) return;
-  const int* bt = block_tables + (int64_t)token_seq[t] * max_blocks;
-  const int64_t p0 = p + 1 - pool;
-  const int64_t page0 = bt[p0 / bs];
-  const int e = (int)((p0 % bs) / pool);
-  for (int d = threadIdx.x; d < D + V; d += 64) {
-    const bool is_k = d < D;
-    const int dd = is_k ? d : d - D;
-    const int W = is_k ? D : V;
-    const AT* cache = is_k ? k_cache : v_cache;
-    float acc = 0.f;
-    for (int j = 0; j < pool; ++j) {
-      const int64_t pos = p0 + j;
-      const int64_t page = bt[pos / bs];
-      acc += Act<AT>::ld(cache + ((page * G + g) * bs + pos % bs) * W + dd);
-    }
-    AT* dst = (is_k ? kp_cache : vp_cache) + ((page0 * G + g) * spp + e) * W + dd;
-    Act<AT>::st(dst, acc / (float)pool);
+    const int* __restrict__ token_seq, int T, int max_blocks, int G, int D,
+    int V, int bs, int pool, int spp) {
+  __shared__ int list_s[64];
+  __shared__ int count_s;
+  const int g = blockIdx.y, tid = threadIdx.x;
+  if (tid == 0) count_s = 0;
+  __syncthreads();
+  if (tid < 64) {
+    const int t = blockIdx.x * 64 + tid;
+    if (t < T && slot_mapping[t] >= 0 && (positions[t] + 1) % pool == 0)
+      list_s[atomicAdd(&count_s, 1)] = t;
   }
+  __syncthreads();
+  const int wave = tid / 64, lane = tid % 64;
+  for (int i = wave; i < count_s; i += 4) {
+    const int t = list_s[i];
+    const int* bt = block_tables + (int64_t)token_seq[t] * max_blocks;
+    const int64_t p0 = positions[t] + 1 - pool;
+    const int64_t page0 = bt[p0 / bs];
+    const int e = (int)((p0 % bs) / pool);
+    for (int d = lane; d < D + V; d += 64) {
+      const bool is_k = d < D;
+      const int dd = is_k ? d : d - D;
+      const int W = is_k ? D : V;
+      const AT* cache = is_k ? k_cache : v_cache;
+      float acc = 0.f;
+      for (int j = 0; j < pool; ++j) {
+        const int64_t pos = p0 + j;
+        const int64_t page = bt[pos / bs];
+        acc += Act<AT>::ld(cache + ((page * G + g) * bs + pos % bs) * W + dd);
+      }
+      AT* dst = (is_k ? kp_cache : vp_cache) + ((page0 * G + g) * spp + e) * W + dd;
+      Act<AT>::st(dst, acc / (float)pool);
+    }
+  }
+}
+
+// q (fp32, LDS) . key row; 16-byte loads when rows are aligned for them
+template <typename AT>
+__device__ __forceinline__ float dot_row(const float* q_s, const AT* kr, int D,
+                                         bool vec);
+template <>
+__device__ __forceinline__ float dot_row<bf16>(const float* q_s, const bf16* kr,
+                                               int D, bool vec) {
+  float dot = 0.f;
+  if (vec) {
+    for (int d = 0; d < D; d += 8) {
+      const ushort8 u = *reinterpret_cast<const ushort8*>(kr + d);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot += q_s[d + e] * bf16_bits_to_float(u[e]);
+    }
+  } else {
+    for (int d = 0; d < D; ++d) dot += q_s[d] * bf16_bits_to_float(kr[d]);
+  }
+  return dot;
+}
+template <>
+__device__ __forceinline__ float dot_row<float>(const float* q_s,
+                                                const float* kr, int D,
+                                                bool vec) {
+  float dot = 0.f;
+  if (vec) {
+    for (int d = 0; d < D; d += 4) {
+      const float4v u = *reinterpret_cast<const float4v*>(kr + d);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dot += q_s[d + e] * u[e];
+    }
+  } else {
+    for (int d = 0; d < D; ++d) dot += q_s[d] * kr[d];
+  }
+  return dot;
 }
 
 constexpr int WP_MAX_D = 512;  // query dims held in LDS
@@ -95,6 +144,7 @@ __global__ __launch_bounds__(64) void attn_window_pool_kernel(
   const int nb = pos - window + 1 > 0 ? (pos - window + 1) / pool : 0;
   const int nkeys = nb + pos - lo + 1;
   const int g = h / (H / G);
+  const bool vec = D % 8 == 0;  // rows of D elements start 16 bytes apart
   const int* bt = block_tables + (int64_t)s * max_blocks;
   for (int d = lane; d < D; d += 64)
     q_s[d] = Act<AT>::ld(q + (int64_t)t * ldq + (int64_t)h * D + d);
@@ -121,9 +171,7 @@ __global__ __launch_bounds__(64) void attn_window_pool_kernel(
         kr = k_cache + e * D;
         vr = v_cache + e * V;
       }
-      float dot = 0.f;
-      for (int d = 0; d < D; ++d) dot += q_s[d] * Act<AT>::ld(kr + d);
-      sc = dot * scale;
+      sc = dot_row<AT>(q_s, kr, D, vec) * scale;
     }
     const float m_new = fmaxf(m, wave_reduce_max(sc));
     const float p = valid ? expf(sc - m_new) : 0.f;
@@ -171,12 +219,12 @@ extern "C" void arks_seq_kv_write_pooled(
     hipLaunchKernelGGL((kv_write_kernel<AT>), dim3(T), dim3(256), 0, stream,
                        (const AT*)k, (const AT*)v, ldk, ldv, (AT*)k_cache,
                        (AT*)v_cache, (const int64_t*)slot_mapping, G, D, V, bs);
-    hipLaunchKernelGGL((kv_pool_kernel<AT>), dim3(T, G), dim3(64), 0, stream,
-                       (const AT*)k_cache, (const AT*)v_cache, (AT*)kp_cache,
-                       (AT*)vp_cache, (const int64_t*)slot_mapping,
-                       (const int64_t*)positions, (const int*)block_tables,
-                       (const int*)token_seq, max_blocks, G, D, V, bs, pool,
-                       spp);
+    hipLaunchKernelGGL((kv_pool_kernel<AT>), dim3((T + 63) / 64, G), dim3(256),
+                       0, stream, (const AT*)k_cache, (const AT*)v_cache,
+                       (AT*)kp_cache, (AT*)vp_cache,
+                       (const int64_t*)slot_mapping, (const int64_t*)positions,
+                       (const int*)block_tables, (const int*)token_seq, T,
+                       max_blocks, G, D, V, bs, pool, spp);
   });
 }
 

@@ -15,7 +15,11 @@
 //   * q/k size and value size are separate template parameters, q and out
 //     are row-strided views, the output is multiplied by out_scale;
 //   * no host work list: workgroup y finds its (sequence, q0) by walking
-//     cu_seqlens, so the launch depends on tensor shapes only.
+//     cu_seqlens, so the launch depends on tensor shapes only;
+//   * DEC (steps of single rows): a workgroup is one (row, key/value head)
+//     and the tile's rows are the query heads that share it, so keys and
+//     values are read once for the whole group; waves without a query head
+//     only help to stage the tiles.
 #include "seq_common.h"
 
 #include <cfloat>
@@ -31,22 +35,25 @@ constexpr int WPM_KTILE = 32;
 constexpr int WPM_PAGE = 16;
 constexpr int WPM_PPAD = 40;
 
-template <int D, int V>
+template <int D, int V, bool DEC>
 __global__ __launch_bounds__(256) void attn_window_pool_mfma_kernel(
     bf16* __restrict__ out, int64_t ldo, const bf16* __restrict__ q,
     int64_t ldq, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, const bf16* __restrict__ kp_cache,
     const bf16* __restrict__ vp_cache, const int* __restrict__ block_tables,
-    const int* __restrict__ kv_lens, const int* __restrict__ cu, int num_seqs,
-    float scale, int window, int pool, int spp, float out_scale, int G,
-    int H, int max_blocks) {
+    const int* __restrict__ kv_lens, const int* __restrict__ cu,
+    const int* __restrict__ token_seq, int num_seqs, float scale, int window,
+    int pool, int spp, float out_scale, int G, int H, int max_blocks) {
   constexpr int STEPS = D / 32;
   constexpr int CHUNKS = V / 16;
   constexpr int SWZ = ((D & (D - 1)) == 0 && D >= 64) ? 1 : 0;
 
   // which q tile is this workgroup's
   int seq_idx = -1, q0 = 0;
-  {
+  if (DEC) {
+    seq_idx = token_seq[blockIdx.y];
+    q0 = blockIdx.y - cu[seq_idx];
+  } else {
     int left = blockIdx.y;
     for (int s = 0; s < num_seqs; ++s) {
       const int n = (cu[s + 1] - cu[s] + WPM_QTILE - 1) / WPM_QTILE;
@@ -59,8 +66,8 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_kernel(
     }
   }
   if (seq_idx < 0) return;
-  const int h = blockIdx.x;
-  const int kvh = h / (H / G);
+  const int GQ = H / G;
+  const int kvh = DEC ? blockIdx.x : blockIdx.x / GQ;
   const int q_start = cu[seq_idx];
   const int q_len = cu[seq_idx + 1] - q_start;
   const int kv_len = kv_lens[seq_idx];
@@ -75,8 +82,12 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_kernel(
   __shared__ __attribute__((aligned(16))) bf16 vt_img[V / 16][8][96];
   __shared__ __attribute__((aligned(16))) bf16 p_lds[4][16][WPM_PPAD];
 
-  const int my_qrow = q0 + wave * 16 + lq;
-  const bool qrow_valid = my_qrow < q_len;
+  // this lane's score column: a row of the sequence, or (DEC) a query head
+  // of the group, all at the one row's position
+  const int my_qrow = DEC ? q0 : q0 + wave * 16 + lq;
+  const bool qrow_valid = DEC ? wave * 16 + lq < GQ : my_qrow < q_len;
+  const int h = DEC ? kvh * GQ + (qrow_valid ? wave * 16 + lq : 0) : blockIdx.x;
+  const bool wave_active = !DEC || wave * 16 < GQ;
   const int my_pos = kv_off + my_qrow;
   // pooled blocks this lane's row sees
   const int my_nb = my_pos - window + 1 > 0 ? (my_pos - window + 1) / pool : 0;
@@ -96,11 +107,12 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_kernel(
 #pragma unroll
   for (int c = 0; c < CHUNKS; ++c) oacc[c] = {0.f, 0.f, 0.f, 0.f};
 
-  const int last_pos = kv_off + min(q0 + WPM_QTILE, q_len) - 1;
+  const int last_pos = DEC ? my_pos : kv_off + min(q0 + WPM_QTILE, q_len) - 1;
   const int nb_max = last_pos - window + 1 > 0 ? (last_pos - window + 1) / pool : 0;
   const int pool_tiles = (nb_max + WPM_KTILE - 1) / WPM_KTILE;
   const int kmax = last_pos + 1;
   const int tok_j0 = max(0, kv_off + q0 - window + 1) / WPM_KTILE;
+  static_assert(WPM_QTILE == 64, "four waves of 16 rows");
   const int tok_tiles = (kmax + WPM_KTILE - 1) / WPM_KTILE;
   const int n_iter = pool_tiles + (tok_tiles - tok_j0);
 
@@ -152,6 +164,7 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_kernel(
     }
     __syncthreads();
 
+    if (wave_active) {
     wp_f32x4 sc[2];
     sc[0] = {0.f, 0.f, 0.f, 0.f};
     sc[1] = {0.f, 0.f, 0.f, 0.f};
@@ -219,8 +232,10 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_kernel(
       for (int r = 0; r < 4; ++r) pk[r] = float_to_bf16_bits(p[sub * 4 + r]);
       *reinterpret_cast<ushort4v*>(&p_lds[wave][lq][sub * 16 + 4 * la]) = pk;
     }
+    }
     __syncthreads();
 
+    if (wave_active) {
     ushort8 pa = *reinterpret_cast<const ushort8*>(&p_lds[wave][lq][8 * la]);
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
@@ -239,6 +254,7 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_kernel(
       oacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
           *reinterpret_cast<wp_bf16x8*>(&pa), vb, oacc[c], 0, 0, 0);
     }
+    }
     __syncthreads();
   }
 
@@ -250,9 +266,11 @@ __global__ __launch_bounds__(256) void attn_window_pool_mfma_kernel(
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int row = q0 + wave * 16 + 4 * la + r;
-    if (row >= q_len) continue;
-    const int64_t obase = (int64_t)(q_start + row) * ldo + (int64_t)h * V;
+    const int sub = wave * 16 + 4 * la + r;  // row of the tile
+    if (DEC ? sub >= GQ : q0 + sub >= q_len) continue;
+    const int64_t obase =
+        DEC ? (int64_t)(q_start + q0) * ldo + (int64_t)(kvh * GQ + sub) * V
+            : (int64_t)(q_start + q0 + sub) * ldo + (int64_t)blockIdx.x * V;
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c)
       out[obase + c * 16 + lq] = float_to_bf16_bits(oacc[c][r] * row_inv[r]);
@@ -271,21 +289,28 @@ extern "C" int arks_seq_attn_window_pool_mfma(
     const void* block_tables, const void* seq_lens, const void* cu,
     const void* token_seq, float scale, int window, int pool, int spp,
     float out_scale, int T, int H, int G, int D, int V, int bs, int max_blocks,
-    int num_seqs, hipStream_t stream) {
-  if (bs != WPM_PAGE || ldq % 8 || H % G) return 1;
+    int num_seqs, int single_rows, hipStream_t stream) {
+  if (bs != WPM_PAGE || ldq % 8 || H % G || ((uintptr_t)q & 15)) return 1;
+  if (single_rows && H / G > WPM_QTILE) return 1;
   if (T == 0) return 0;
-  // every sequence adds at most one partly filled tile
+  // prompts: every sequence adds at most one partly filled tile
   dim3 grid(H, (T + WPM_QTILE - 1) / WPM_QTILE + num_seqs), block(256);
+  if (single_rows) grid = dim3(G, T);
+#define WPM_ARGS                                                              \
+  grid, block, 0, stream, (bf16*)out, ldo, (const bf16*)q, ldq,               \
+      (const bf16*)k_cache, (const bf16*)v_cache, (const bf16*)kp_cache,      \
+      (const bf16*)vp_cache, (const int*)block_tables, (const int*)seq_lens,  \
+      (const int*)cu, (const int*)token_seq, num_seqs, scale, window, pool,   \
+      spp, out_scale, G, H, max_blocks
 #define WPM(DD, VV)                                                           \
   if (D == DD && V == VV) {                                                   \
-    hipLaunchKernelGGL((attn_window_pool_mfma_kernel<DD, VV>), grid, block,   \
-                       0, stream, (bf16*)out, ldo, (const bf16*)q, ldq,        \
-                       (const bf16*)k_cache, (const bf16*)v_cache,             \
-                       (const bf16*)kp_cache, (const bf16*)vp_cache,           \
-                       (const int*)block_tables, (const int*)seq_lens,         \
-                       (const int*)cu, num_seqs, scale, window, pool, spp,     \
-                       out_scale, G, H, max_blocks);                           \
-    return 0;                                                                  \
+    if (single_rows)                                                          \
+      hipLaunchKernelGGL((attn_window_pool_mfma_kernel<DD, VV, true>),        \
+                         WPM_ARGS);                                           \
+    else                                                                      \
+      hipLaunchKernelGGL((attn_window_pool_mfma_kernel<DD, VV, false>),       \
+                         WPM_ARGS);                                           \
+    return 0;                                                                 \
   }
   WPM(64, 64)
   WPM(128, 128)
@@ -294,5 +319,6 @@ extern "C" int arks_seq_attn_window_pool_mfma(
   WPM(32, 32)
   WPM(96, 96)
 #undef WPM
+#undef WPM_ARGS
   return 1;
 }

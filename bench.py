@@ -55,7 +55,10 @@ def parse_args():
     # model cut to the same width and depth, one JSON line per model and
     # phase. --design-only NAME runs one of the two (profiling).
     p.add_argument("--design-bench", action="store_true")
-    p.add_argument("--design-only", choices=["gagorax", "llama"], default=None)
+    p.add_argument("--design-only", choices=["gagorax", "fusolix", "llama"],
+                   default=None)
+    # which layer-list design --design-bench measures beside llama
+    p.add_argument("--design", choices=["gagorax", "fusolix"], default="gagorax")
     p.add_argument("--cold-start", action="store_true")
     p.add_argument("--ckpt-dir", default="/tmp/arks_ckpt")
     return p.parse_args()
@@ -126,10 +129,11 @@ def run_cold_start(args):
 
 
 def run_design_bench(args):
-    """Gagorax (8 blocks at the sizes of an 8B model) against llama-3-8b cut
-    to 8 layers: prefill tokens/s for one long prompt and for a batch of
-    prompts, decode tokens/s for a batch at a fixed context. Random weights,
-    synthetic tokens, one GPU."""
+    """A layer-list design (--design: Gagorax or Fusolix, 8 blocks at the
+    sizes of an 8B model) against llama-3-8b cut to 8 layers: prefill
+    tokens/s for one long prompt and for a batch of prompts, decode tokens/s
+    for a batch at a fixed context. Random weights, synthetic tokens, one
+    GPU."""
     import dataclasses
 
     from arks_amd.config import EngineConfig, PRESET_CONFIGS
@@ -138,7 +142,7 @@ def run_design_bench(args):
     PRESET_CONFIGS["llama-3-8b-8l"] = dataclasses.replace(
         PRESET_CONFIGS["llama-3-8b"], num_hidden_layers=8)
     use_gpu = torch.cuda.is_available()
-    models = {"gagorax": "gagorax-8b-slice", "llama": "llama-3-8b-8l"}
+    models = {args.design: args.design + "-8b-slice", "llama": "llama-3-8b-8l"}
     prefills = [(1, 8192), (8, 2048), (32, 128)]  # (prompts, tokens each)
     dec_batch, dec_ctx = args.batch, args.input_len
     for key, preset in models.items():
