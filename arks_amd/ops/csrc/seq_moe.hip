@@ -120,6 +120,31 @@ __global__ __launch_bounds__(256) void moe_mix_rows_kernel(
   }
 }
 
+// bf16, 8 channels per thread (H % 8 == 0)
+__global__ __launch_bounds__(256) void moe_mix_rows_vec8_kernel(
+    bf16* __restrict__ out, const bf16* __restrict__ y,
+    const float* __restrict__ weights, const int* __restrict__ rows, int T,
+    int H, int k, int dense) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x * 8; c < H; c += 256 * 8) {
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int j = 0; j < k; ++j) {
+      const int64_t r = dense ? (int64_t)rows[t * k + j] * T + t
+                              : (int64_t)rows[t * k + j];
+      const float w = weights[t * k + j];
+      const ushort8 u = *reinterpret_cast<const ushort8*>(y + r * H + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += w * bf16_bits_to_float(u[e]);
+    }
+    ushort8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = float_to_bf16_bits(acc[e]);
+    *reinterpret_cast<ushort8*>(out + (int64_t)t * H + c) = o;
+  }
+}
+
 }  // namespace arks
 
 using namespace arks;
@@ -143,6 +168,12 @@ extern "C" void arks_seq_moe_mix_rows(void* out, const void* y,
                                       int T, int H, int k, int dense,
                                       int act_f32, hipStream_t stream) {
   if (T == 0) return;
+  if (!act_f32 && H % 8 == 0) {
+    hipLaunchKernelGGL(moe_mix_rows_vec8_kernel, dim3(T), dim3(256), 0, stream,
+                       (bf16*)out, (const bf16*)y, (const float*)weights,
+                       (const int*)rows, T, H, k, dense);
+    return;
+  }
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
       (moe_mix_rows_kernel<AT>), dim3(T), dim3(256), 0, stream, (AT*)out,
       (const AT*)y, (const float*)weights, (const int*)rows, T, H, k, dense));

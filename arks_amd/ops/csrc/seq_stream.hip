@@ -117,6 +117,89 @@ __global__ __launch_bounds__(256) void stream_mix_norm_kernel(
     n_out[t * C + c] = (u_s[c] - mean) * rstd * norm_w[c] + norm_b[c];
 }
 
+// The same for S <= 4 copies and rows of up to 1024 * NV channels
+// (C % 4 == 0): every thread keeps its float4 pieces of u in registers
+// between the passes, so the copies are read once and nothing is staged.
+template <typename AT, int NV, int S>
+__global__ __launch_bounds__(256) void stream_mix_norm_reg_kernel(
+    float* __restrict__ xs, float* __restrict__ n_out,
+    const AT* __restrict__ y, int64_t ldy, const float* __restrict__ y_bias,
+    const float* __restrict__ mix, const float* __restrict__ out_w,
+    const float* __restrict__ in_w, const float* __restrict__ norm_w,
+    const float* __restrict__ norm_b, float eps, int64_t T, int C) {
+  __shared__ float red[8];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x;
+  float mixv[S * S], outv[S], inv_[S];
+#pragma unroll
+  for (int i = 0; i < S * S; ++i) mixv[i] = y ? mix[i] : 0.f;
+#pragma unroll
+  for (int i = 0; i < S; ++i) {
+    outv[i] = y ? out_w[i] : 0.f;
+    inv_[i] = in_w ? in_w[i] : 0.f;
+  }
+  float4v u[NV];
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = (tid + 256 * j) * 4;
+    u[j] = {0.f, 0.f, 0.f, 0.f};
+    if (c < C) {
+      float4v old[S];
+#pragma unroll
+      for (int s = 0; s < S; ++s)
+        old[s] = *reinterpret_cast<const float4v*>(xs + ((int64_t)s * T + t) * C + c);
+      if (y) {
+        float4v yv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) yv[e] = Act<AT>::ld(y + t * ldy + c + e);
+        if (y_bias) yv += *reinterpret_cast<const float4v*>(y_bias + c);
+#pragma unroll
+        for (int d = 0; d < S; ++d) {
+          float4v nw = outv[d] * yv;
+#pragma unroll
+          for (int s = 0; s < S; ++s) nw += mixv[s * S + d] * old[s];
+          *reinterpret_cast<float4v*>(xs + ((int64_t)d * T + t) * C + c) = nw;
+          u[j] += inv_[d] * nw;
+        }
+      } else {
+#pragma unroll
+        for (int d = 0; d < S; ++d) u[j] += inv_[d] * old[d];
+      }
+      sum += u[j][0] + u[j][1] + u[j][2] + u[j][3];
+    }
+  }
+  if (!in_w) return;
+  const float mean = block_reduce_sum<256>(sum, red) / (float)C;
+  __syncthreads();
+  float sq = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = (tid + 256 * j) * 4;
+    if (c < C) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float d = u[j][e] - mean;
+        sq += d * d;
+      }
+    }
+  }
+  const float var = block_reduce_sum<256>(sq, red) / (float)C;
+  const float rstd = 1.f / sqrtf(var + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = (tid + 256 * j) * 4;
+    if (c < C) {
+      const float4v w = *reinterpret_cast<const float4v*>(norm_w + c);
+      const float4v b = *reinterpret_cast<const float4v*>(norm_b + c);
+      float4v o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (u[j][e] - mean) * rstd * w[e] + b[e];
+      *reinterpret_cast<float4v*>(n_out + t * C + c) = o;
+    }
+  }
+}
+
 // One block per (row, 256 channels). Inputs before the step's first row come
 // from the sequence's stored history (zeros at position 0); the history is
 // replaced by a later launch, so every reader here sees the old one.
@@ -146,6 +229,75 @@ __global__ __launch_bounds__(256) void short_conv_residual_kernel(
     acc += w[(int64_t)c * taps + j] * xv;
   }
   Act<AT>::st(out + (int64_t)t * C + c, acc);
+}
+
+// 4 channels per thread and rpb consecutive rows per block (16 for long
+// steps, fewer for short ones so the grid still fills the chip): the thread
+// walks its rows with the last taps-1 inputs in registers, so every input
+// is read once per block (plus the block's first rows' history).
+constexpr int SC_MAX_TAPS = 8;
+
+template <typename AT>
+__global__ __launch_bounds__(256) void short_conv_residual_vec_kernel(
+    AT* __restrict__ out, const float* __restrict__ h,
+    const float* __restrict__ w, const float* __restrict__ state,
+    const int* __restrict__ cu, const int* __restrict__ seq_lens,
+    const int* __restrict__ slots, const int* __restrict__ token_seq, int T,
+    int C, int taps, int rpb) {
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+  if (c >= C) return;
+  float4v wv[SC_MAX_TAPS];
+#pragma unroll
+  for (int j = 0; j < SC_MAX_TAPS; ++j)
+    if (j < taps) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) wv[j][e] = w[(int64_t)(c + e) * taps + j];
+    }
+  const int t0 = blockIdx.x * rpb;
+  const int t1 = min(T, t0 + rpb);
+  float4v prev[SC_MAX_TAPS];  // prev[j]: the input taps-1-j rows back
+  int cur_seq = -1;
+  for (int t = t0; t < t1; ++t) {
+    const int seq = token_seq[t];
+    if (seq != cur_seq) {
+      // (re)load the history of this row: earlier rows of the step, the
+      // sequence's stored inputs, or zeros before its start
+      cur_seq = seq;
+      const SeqRow r = seq_row(t, token_seq, cu, seq_lens, slots);
+      const int i = t - r.first_row;
+      const bool has_state = r.start > 0 && r.slot >= 0;
+      const float* hist =
+          state ? state + (int64_t)(r.slot < 0 ? 0 : r.slot) * (taps - 1) * C : nullptr;
+#pragma unroll
+      for (int j = 0; j < SC_MAX_TAPS; ++j)
+        if (j < taps - 1) {
+          const int src = i - (taps - 1 - j);
+          if (src >= 0)
+            prev[j] = *reinterpret_cast<const float4v*>(
+                h + (int64_t)(r.first_row + src) * C + c);
+          else if (has_state)
+            prev[j] = *reinterpret_cast<const float4v*>(
+                hist + (int64_t)(src + taps - 1) * C + c);
+          else
+            prev[j] = {0.f, 0.f, 0.f, 0.f};
+        }
+    }
+    const float4v x = *reinterpret_cast<const float4v*>(h + (int64_t)t * C + c);
+    float4v acc = x;
+#pragma unroll
+    for (int j = 0; j < SC_MAX_TAPS; ++j)
+      if (j < taps - 1) acc += wv[j] * prev[j];
+#pragma unroll
+    for (int j = 0; j < SC_MAX_TAPS; ++j)
+      if (j == taps - 1) acc += wv[j] * x;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) Act<AT>::st(out + (int64_t)t * C + c + e, acc[e]);
+#pragma unroll
+    for (int j = 0; j < SC_MAX_TAPS - 1; ++j) {
+      if (j < taps - 2) prev[j] = prev[j + 1];
+      else if (j == taps - 2) prev[j] = x;
+    }
+  }
 }
 
 constexpr int SC_MAX_HIST = 15;
@@ -261,6 +413,29 @@ extern "C" int arks_seq_stream_mix_norm(
   if (T == 0) return 0;
   const size_t lds = (size_t)C * 4;
   const bool vec = C % 4 == 0 && (y == nullptr || ldy % 4 == 0);
+  if (C % 4 == 0 && C <= 8192 && S <= 4) {
+#define SMR(NV, SS)                                                            \
+  SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(                                \
+      (stream_mix_norm_reg_kernel<AT, NV, SS>), dim3((unsigned)T), dim3(256),  \
+      0, stream, (float*)xs, (float*)n_out, (const AT*)y, ldy,                 \
+      (const float*)y_bias, (const float*)mix, (const float*)out_w,            \
+      (const float*)in_w, (const float*)norm_w, (const float*)norm_b, eps, T,  \
+      C))
+#define SMS(NV)                \
+  do {                         \
+    if (S == 1) SMR(NV, 1);    \
+    else if (S == 2) SMR(NV, 2); \
+    else if (S == 3) SMR(NV, 3); \
+    else SMR(NV, 4);           \
+  } while (0)
+    if (C <= 1024) SMS(1);
+    else if (C <= 2048) SMS(2);
+    else if (C <= 4096) SMS(4);
+    else SMS(8);
+#undef SMS
+#undef SMR
+    return 0;
+  }
 #define SMN(VEC)                                                              \
   SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(                               \
       (stream_mix_norm_kernel<AT, VEC>), dim3((unsigned)T), dim3(256), lds,   \
@@ -281,11 +456,21 @@ extern "C" int arks_seq_short_conv_residual(
   if (taps - 1 > SC_MAX_HIST) return 1;
   if (T == 0) return 0;
   const int cb = (C + 255) / 256;
-  SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
-      (short_conv_residual_kernel<AT>), dim3(T, cb), dim3(256), 0, stream,
-      (AT*)out, (const float*)h, (const float*)w, (const float*)state,
-      (const int*)cu, (const int*)seq_lens, (const int*)slots,
-      (const int*)token_seq, C, taps));
+  if (C % 4 == 0 && taps <= SC_MAX_TAPS) {
+    const int rpb = T >= 8192 ? 16 : (T >= 1024 ? 4 : 1);
+    SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
+        (short_conv_residual_vec_kernel<AT>),
+        dim3((T + rpb - 1) / rpb, (C / 4 + 255) / 256), dim3(256), 0,
+        stream, (AT*)out, (const float*)h, (const float*)w,
+        (const float*)state, (const int*)cu, (const int*)seq_lens,
+        (const int*)slots, (const int*)token_seq, T, C, taps, rpb));
+  } else {
+    SEQ_DISPATCH_ACT(act_f32, hipLaunchKernelGGL(
+        (short_conv_residual_kernel<AT>), dim3(T, cb), dim3(256), 0, stream,
+        (AT*)out, (const float*)h, (const float*)w, (const float*)state,
+        (const int*)cu, (const int*)seq_lens, (const int*)slots,
+        (const int*)token_seq, C, taps));
+  }
   if (taps > 1)
     hipLaunchKernelGGL(short_conv_state_kernel, dim3(S, cb), dim3(256), 0,
                        stream, (float*)state, (const float*)h, (const int*)cu,

@@ -81,6 +81,64 @@ __global__ __launch_bounds__(256) void kv_pool_kernel(
   }
 }
 
+// bf16 pages whose key + value dims make NC = (D + V) / 8 16-byte pieces with
+// 64 % NC == 0: lane = (piece, position group); every lane sums its group's
+// positions of its piece, the groups meet through shuffles.
+__global__ __launch_bounds__(256) void kv_pool_vec_kernel(
+    const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    bf16* __restrict__ kp_cache, bf16* __restrict__ vp_cache,
+    const int64_t* __restrict__ slot_mapping,
+    const int64_t* __restrict__ positions, const int* __restrict__ block_tables,
+    const int* __restrict__ token_seq, int T, int max_blocks, int G, int D,
+    int V, int bs, int pool, int spp) {
+  __shared__ int list_s[64];
+  __shared__ int count_s;
+  const int g = blockIdx.y, tid = threadIdx.x;
+  if (tid == 0) count_s = 0;
+  __syncthreads();
+  if (tid < 64) {
+    const int t = blockIdx.x * 64 + tid;
+    if (t < T && slot_mapping[t] >= 0 && (positions[t] + 1) % pool == 0)
+      list_s[atomicAdd(&count_s, 1)] = t;
+  }
+  __syncthreads();
+  const int wave = tid / 64, lane = tid % 64;
+  const int nc = (D + V) / 8, groups = 64 / nc;
+  const int piece = lane % nc, grp = lane / nc;
+  const bool is_k = piece * 8 < D;
+  const int dd = is_k ? piece * 8 : piece * 8 - D;
+  const int W = is_k ? D : V;
+  const bf16* cache = is_k ? k_cache : v_cache;
+  for (int i = wave; i < count_s; i += 4) {
+    const int t = list_s[i];
+    const int* bt = block_tables + (int64_t)token_seq[t] * max_blocks;
+    const int64_t p0 = positions[t] + 1 - pool;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int j = grp; j < pool; j += groups) {
+      const int64_t pos = p0 + j;
+      const int64_t page = bt[pos / bs];
+      const ushort8 u = *reinterpret_cast<const ushort8*>(
+          cache + ((page * G + g) * bs + pos % bs) * W + dd);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += bf16_bits_to_float(u[e]);
+    }
+    for (int off = nc; off < 64; off <<= 1)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] += __shfl_xor(acc[e], off, 64);
+    if (grp == 0) {
+      const int64_t page0 = bt[p0 / bs];
+      const int e0 = (int)((p0 % bs) / pool);
+      ushort8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] = float_to_bf16_bits(acc[e] / (float)pool);
+      *reinterpret_cast<ushort8*>((is_k ? kp_cache : vp_cache) +
+                                  ((page0 * G + g) * spp + e0) * W + dd) = o;
+    }
+  }
+}
+
 // q (fp32, LDS) . key row; 16-byte loads when rows are aligned for them
 template <typename AT>
 __device__ __forceinline__ float dot_row(const float* q_s, const AT* kr, int D,
@@ -215,6 +273,19 @@ extern "C" void arks_seq_kv_write_pooled(
     int T, int max_blocks, int G, int D, int V, int bs, int pool, int spp,
     int act_f32, hipStream_t stream) {
   if (T == 0) return;
+  const int nc = (D + V) / 8;
+  if (!act_f32 && D % 8 == 0 && V % 8 == 0 && nc <= 64 && 64 % nc == 0) {
+    hipLaunchKernelGGL((kv_write_kernel<bf16>), dim3(T), dim3(256), 0, stream,
+                       (const bf16*)k, (const bf16*)v, ldk, ldv, (bf16*)k_cache,
+                       (bf16*)v_cache, (const int64_t*)slot_mapping, G, D, V, bs);
+    hipLaunchKernelGGL(kv_pool_vec_kernel, dim3((T + 63) / 64, G), dim3(256), 0,
+                       stream, (const bf16*)k_cache, (const bf16*)v_cache,
+                       (bf16*)kp_cache, (bf16*)vp_cache,
+                       (const int64_t*)slot_mapping, (const int64_t*)positions,
+                       (const int*)block_tables, (const int*)token_seq, T,
+                       max_blocks, G, D, V, bs, pool, spp);
+    return;
+  }
   SEQ_DISPATCH_ACT(act_f32, {
     hipLaunchKernelGGL((kv_write_kernel<AT>), dim3(T), dim3(256), 0, stream,
                        (const AT*)k, (const AT*)v, ldk, ldv, (AT*)k_cache,

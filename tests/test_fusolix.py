@@ -226,7 +226,9 @@ OTHER_SIZES = {
                                  r_heads=3, r_dim=12, r_vdim=20, rot_dims=4,
                                  decay=(0.5, 0.999, 1.0), width=40,
                                  layers=("dense",)),
-    "full-rotary-no-rotary": dict(rot_dims=16, layers=(None,)),
+    "odd-left-dims": dict(heads=2, kv_heads=1, dim=12, vdim=20, width=36,
+                          layers=(None,)),
+    "full-rotary": dict(rot_dims=16, layers=(None,)),
     "no-rotary": dict(rot_dims=0, layers=(None,)),
     "every-group-kept-top-one": dict(experts=8, groups=4, keep=4, top=1,
                                      layers=("moe",)),
@@ -346,8 +348,9 @@ def test_stream_mix_norm(device, dtype, streams):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
-@pytest.mark.parametrize("taps", [1, 2, 4, 6])
-def test_short_conv_portions(device, dtype, taps):
+@pytest.mark.parametrize("taps,C", [(1, 40), (2, 40), (4, 40), (6, 42),
+                                    (10, 40)])
+def test_short_conv_portions(device, dtype, taps, C):
     """Two sequences in portions of 1, 2 and more rows sharing steps; the
     history crosses every portion edge; slots hold another sequence's
     leftovers first."""
@@ -355,7 +358,6 @@ def test_short_conv_portions(device, dtype, taps):
 
     dev = _dev(device)
     g = torch.Generator().manual_seed(taps)
-    C = 40
     w = torch.randn(C, taps, generator=g, dtype=F64)
     seqs = [torch.randn(n, C, generator=g, dtype=F64) for n in (23, 9)]
     want = [O.short_conv_residual(h, w) for h in seqs]
