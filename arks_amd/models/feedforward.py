@@ -13,8 +13,8 @@ constants as constructor parameters:
   framework's other sparse feed-forward (models/llama_family.py MoEMLP), and
   the two execution paths are the same: below DENSE_TOKENS rows every expert
   runs on every row as two batched GEMMs (data-independent shapes, so the
-  step can be captured), above it rows are sorted by expert and run as a
-  capacity-padded batched GEMM.
+  step can be captured), above it the (row, expert) pairs are sorted by
+  expert and every expert runs plain GEMMs on its own segment.
 """
 
 from __future__ import annotations
@@ -79,25 +79,30 @@ class GroupedMoE(nn.Module):
             a = ops.glu_act(gu.view(E * T, 2 * ff), "swiglu")
             y = torch.bmm(a.view(E, T, ff), self.w2)
             return ops.moe_mix_seq(y, weights, ids)
-        # rows sorted by expert, every expert's segment padded to the
-        # heaviest one's length (one host read of the segment table)
+        # (row, expert) pairs sorted by expert: every expert runs two plain
+        # GEMMs on its own contiguous segment, nothing is padded (one host
+        # read of the segment sizes)
         flat = ids.reshape(-1).long()
         order = torch.argsort(flat, stable=True)
         tok = torch.div(order, k, rounding_mode="floor")
-        counts = torch.bincount(flat, minlength=E)
-        starts = torch.cumsum(counts, 0) - counts
-        cap = int(counts.max())
-        ar = torch.arange(cap, device=h.device)[None, :]
-        src = torch.where(ar < counts[:, None], starts[:, None] + ar,
-                          torch.zeros_like(ar)).reshape(-1)
-        xp = h[tok[src]].view(E, cap, W)
-        gu = torch.bmm(xp, self.w13)
-        a = ops.glu_act(gu.view(E * cap, 2 * ff), "swiglu")
-        y = torch.bmm(a.view(E, cap, ff), self.w2).view(E * cap, W)
+        counts = torch.bincount(flat, minlength=E).tolist()
+        xs = h[tok]
+        gu = torch.empty((T * k, 2 * ff), dtype=h.dtype, device=h.device)
+        at = 0
+        for e, n in enumerate(counts):
+            if n:
+                torch.mm(xs[at:at + n], self.w13[e], out=gu[at:at + n])
+            at += n
+        a = ops.glu_act(gu, "swiglu")
+        y = torch.empty((T * k, W), dtype=h.dtype, device=h.device)
+        at = 0
+        for e, n in enumerate(counts):
+            if n:
+                torch.mm(a[at:at + n], self.w2[e], out=y[at:at + n])
+            at += n
         inv = torch.empty_like(order)
         inv[order] = torch.arange(T * k, device=h.device)
-        rows = flat * cap + (inv - starts[flat])
-        return ops.moe_mix_rows_seq(y, weights, rows.view(T, k).to(torch.int32))
+        return ops.moe_mix_rows_seq(y, weights, inv.view(T, k).to(torch.int32))
 
 
 def build_feedforward(mlp: dict, width: int, dtype) -> nn.Module:

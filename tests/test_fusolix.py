@@ -277,6 +277,28 @@ def test_matrix_core_sizes(tmp_path, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", CASES)
+def test_experts_rows_sorted_by_expert(tmp_path, device, dtype, monkeypatch):
+    """Steps above GroupedMoE.DENSE_TOKENS sort rows by expert and pad every
+    expert's segment; forced here for small steps, beside single tokens
+    that still take the all-experts path."""
+    from arks_amd.models.feedforward import GroupedMoE
+
+    monkeypatch.setattr(GroupedMoE, "DENSE_TOKENS", 3)
+    cfg = O.make_config(layers=("moe", "moe"), experts=9, groups=3, keep=2, top=3)
+    w = write_checkpoint(tmp_path / "m", cfg, seed=2)
+    reqs = {"a": toks(50, seed=1), "b": toks(21, seed=2)}
+    want = {c: oracle_logits(cfg, w, t) for c, t in reqs.items()}
+    a, b = reqs["a"], reqs["b"]
+    steps = [[("a", a[:30], False), ("b", b[:1], False)],
+             [("a", a[30:32], False), ("b", b[1:2], False)],
+             [("a", a[32:], True), ("b", b[2:], True)]]
+    eng = make_engine(tmp_path / "m", device, dtype)
+    got = replay(eng, tmp_path, steps)
+    for c in reqs:
+        assert rel_err(got[c], want[c], routed(cfg, dtype)) < TOL[dtype], c
+
+
+@pytest.mark.parametrize("device,dtype", CASES)
 def test_greedy_generation(tmp_path, device, dtype):
     """LLMEngine.generate (scheduler, sampler, captured decode steps on the
     GPU) picks the oracle's tokens; three prompts share the batch."""
