@@ -50,6 +50,28 @@ __device__ __forceinline__ float lm_load(const bf16* row, int d, int64_t t,
   return first ? x * cs - y * sn : x * cs + y * sn;
 }
 
+// MODE 1 staging walks a head row in pairs so that one sine/cosine serves
+// both dims of a pair (and q and k of the row): pair p < n_rot is a rotary
+// pair, later pairs are two neighbouring plain dims.
+__device__ __forceinline__ void lm_pair_dims(const LmRot& rot, int p, int& d0,
+                                             int& d1) {
+  if (p < rot.n_rot) {
+    d0 = rot.interleaved ? 2 * p : p;
+    d1 = rot.interleaved ? 2 * p + 1 : p + rot.n_rot;
+  } else {
+    d0 = 2 * p;
+    d1 = 2 * p + 1;
+  }
+}
+
+__device__ __forceinline__ void lm_turn(const bf16* row, int d0, int d1,
+                                        float cs, float sn, float& x0,
+                                        float& x1) {
+  const float a = bf16_bits_to_float(row[d0]), b = bf16_bits_to_float(row[d1]);
+  x0 = a * cs - b * sn;
+  x1 = b * cs + a * sn;
+}
+
 typedef __attribute__((ext_vector_type(8))) __bf16 lm_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float lm_f32x4;
 
@@ -99,14 +121,34 @@ __global__ __launch_bounds__(256) void lightning_state_mfma_kernel(
   const int row0 = cu[ch], n = cu[ch + 1] - row0;
   const float l2 = log2f(decay[h]);
   const int tid = threadIdx.x;
-  for (int i = tid; i < LM_ROWS * D; i += 256) {
-    const int j = i / D, d = i - j * D;
-    float x = 0.f;
-    if (j < n)
-      x = lm_load<MODE>(k + (int64_t)(row0 + j) * ldk + (int64_t)h * D, d,
-                        row0 + j, rot) *
-          (MODE == 0 ? 1.f : rot.k_scale) * decay_pow(l2, n - 1 - j);
-    split_bf16(x, kt_hi[d * LK + j], kt_lo[d * LK + j]);
+  if (MODE == 0) {
+    for (int i = tid; i < LM_ROWS * D; i += 256) {
+      const int j = i / D, d = i - j * D;
+      float x = 0.f;
+      if (j < n)
+        x = lm_load<0>(k + (int64_t)(row0 + j) * ldk + (int64_t)h * D, d,
+                       row0 + j, rot) * decay_pow(l2, n - 1 - j);
+      split_bf16(x, kt_hi[d * LK + j], kt_lo[d * LK + j]);
+    }
+  } else {
+    for (int i = tid; i < LM_ROWS * (D / 2); i += 256) {
+      const int j = i / (D / 2), p = i - j * (D / 2);
+      int d0, d1;
+      lm_pair_dims(rot, p, d0, d1);
+      float x0 = 0.f, x1 = 0.f;
+      if (j < n) {
+        float sn = 0.f, cs = 1.f;
+        if (p < rot.n_rot)
+          sincosf((float)rot.positions[row0 + j] * rot.freq[p], &sn, &cs);
+        lm_turn(k + (int64_t)(row0 + j) * ldk + (int64_t)h * D, d0, d1, cs, sn,
+                x0, x1);
+        const float f = rot.k_scale * decay_pow(l2, n - 1 - j);
+        x0 *= f;
+        x1 *= f;
+      }
+      split_bf16(x0, kt_hi[d0 * LK + j], kt_lo[d0 * LK + j]);
+      split_bf16(x1, kt_hi[d1 * LK + j], kt_lo[d1 * LK + j]);
+    }
   }
   for (int i = tid; i < LM_ROWS * V; i += 256) {
     const int j = i / V, c = i - j * V;
@@ -167,17 +209,41 @@ __global__ __launch_bounds__(256) void lightning_out_mfma_kernel(
   const int row0 = cu[ch], n = cu[ch + 1] - row0;
   const float l2 = log2f(decay[h]);
   const int tid = threadIdx.x;
-  for (int i = tid; i < LM_ROWS * D; i += 256) {
-    const int j = i / D, d = i - j * D;
-    float xq = 0.f, xk = 0.f;
-    if (j < n) {
-      xq = lm_load<MODE>(q + (int64_t)(row0 + j) * ldq + (int64_t)h * D, d,
-                         row0 + j, rot);
-      xk = lm_load<MODE>(k + (int64_t)(row0 + j) * ldk + (int64_t)h * D, d,
-                         row0 + j, rot) * (MODE == 0 ? 1.f : rot.k_scale);
+  if (MODE == 0) {
+    for (int i = tid; i < LM_ROWS * D; i += 256) {
+      const int j = i / D, d = i - j * D;
+      float xq = 0.f, xk = 0.f;
+      if (j < n) {
+        xq = lm_load<0>(q + (int64_t)(row0 + j) * ldq + (int64_t)h * D, d,
+                        row0 + j, rot);
+        xk = lm_load<0>(k + (int64_t)(row0 + j) * ldk + (int64_t)h * D, d,
+                        row0 + j, rot);
+      }
+      qs[j * LD + d] = float_to_bf16_bits(xq);
+      ks[j * LD + d] = float_to_bf16_bits(xk);
     }
-    qs[j * LD + d] = float_to_bf16_bits(xq);
-    ks[j * LD + d] = float_to_bf16_bits(xk);
+  } else {
+    for (int i = tid; i < LM_ROWS * (D / 2); i += 256) {
+      const int j = i / (D / 2), p = i - j * (D / 2);
+      int d0, d1;
+      lm_pair_dims(rot, p, d0, d1);
+      float q0 = 0.f, q1 = 0.f, k0 = 0.f, k1 = 0.f;
+      if (j < n) {
+        float sn = 0.f, cs = 1.f;
+        if (p < rot.n_rot)
+          sincosf((float)rot.positions[row0 + j] * rot.freq[p], &sn, &cs);
+        lm_turn(q + (int64_t)(row0 + j) * ldq + (int64_t)h * D, d0, d1, cs, sn,
+                q0, q1);
+        lm_turn(k + (int64_t)(row0 + j) * ldk + (int64_t)h * D, d0, d1, cs, sn,
+                k0, k1);
+        k0 *= rot.k_scale;
+        k1 *= rot.k_scale;
+      }
+      qs[j * LD + d0] = float_to_bf16_bits(q0);
+      qs[j * LD + d1] = float_to_bf16_bits(q1);
+      ks[j * LD + d0] = float_to_bf16_bits(k0);
+      ks[j * LD + d1] = float_to_bf16_bits(k1);
+    }
   }
   for (int i = tid; i < LM_ROWS * V; i += 256) {
     const int j = i / V, c = i - j * V;

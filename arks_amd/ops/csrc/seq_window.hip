@@ -34,6 +34,29 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
   }
 }
 
+// bf16 rows whose heads are whole 16-byte pieces: one piece per thread.
+__global__ __launch_bounds__(256) void kv_write_vec_kernel(
+    const bf16* __restrict__ k, const bf16* __restrict__ v, int64_t ldk,
+    int64_t ldv, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
+    const int64_t* __restrict__ slot_mapping, int G, int D, int V, int bs) {
+  const int t = blockIdx.x;
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0) return;
+  const int64_t page = slot / bs;
+  const int off = (int)(slot % bs);
+  const int nk = G * D / 8, nv = G * V / 8;
+  for (int i = threadIdx.x; i < nk + nv; i += 256) {
+    const bool is_k = i < nk;
+    const int e = (is_k ? i : i - nk) * 8;
+    const int W = is_k ? D : V;
+    const int g = e / W, d = e - g * W;
+    const ushort8 u = *reinterpret_cast<const ushort8*>(
+        (is_k ? k + (int64_t)t * ldk : v + (int64_t)t * ldv) + e);
+    *reinterpret_cast<ushort8*>((is_k ? k_cache : v_cache) +
+                                ((page * G + g) * bs + off) * W + d) = u;
+  }
+}
+
 // One block per (64 rows, kv head): the rows whose position ends a block are
 // listed first (one in `pool` of a prompt's rows), then the block's waves
 // share them, lanes over the key and value dims. Runs after kv_write_kernel
@@ -116,6 +139,7 @@ __global__ __launch_bounds__(256) void kv_pool_vec_kernel(
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll 4
     for (int j = grp; j < pool; j += groups) {
       const int64_t pos = p0 + j;
       const int64_t page = bt[pos / bs];
@@ -275,9 +299,17 @@ extern "C" void arks_seq_kv_write_pooled(
   if (T == 0) return;
   const int nc = (D + V) / 8;
   if (!act_f32 && D % 8 == 0 && V % 8 == 0 && nc <= 64 && 64 % nc == 0) {
-    hipLaunchKernelGGL((kv_write_kernel<bf16>), dim3(T), dim3(256), 0, stream,
-                       (const bf16*)k, (const bf16*)v, ldk, ldv, (bf16*)k_cache,
-                       (bf16*)v_cache, (const int64_t*)slot_mapping, G, D, V, bs);
+    if (ldk % 8 == 0 && ldv % 8 == 0 &&
+        (((uintptr_t)k | (uintptr_t)v) & 15) == 0)
+      hipLaunchKernelGGL(kv_write_vec_kernel, dim3(T), dim3(256), 0, stream,
+                         (const bf16*)k, (const bf16*)v, ldk, ldv,
+                         (bf16*)k_cache, (bf16*)v_cache,
+                         (const int64_t*)slot_mapping, G, D, V, bs);
+    else
+      hipLaunchKernelGGL((kv_write_kernel<bf16>), dim3(T), dim3(256), 0, stream,
+                         (const bf16*)k, (const bf16*)v, ldk, ldv,
+                         (bf16*)k_cache, (bf16*)v_cache,
+                         (const int64_t*)slot_mapping, G, D, V, bs);
     hipLaunchKernelGGL(kv_pool_vec_kernel, dim3((T + 63) / 64, G), dim3(256), 0,
                        stream, (const bf16*)k_cache, (const bf16*)v_cache,
                        (bf16*)kp_cache, (bf16*)vp_cache,
