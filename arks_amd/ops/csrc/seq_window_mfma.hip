@@ -349,14 +349,16 @@ __global__ __launch_bounds__(256) void attn_window_pool_dec_kernel(
   };
   constexpr int NV = WPM_KTILE * V / 8 / WAVE_SIZE;
 
-  for (int it = wave; it < n_iter; it += 4) {
+  // tile `it` of this wave's keys into registers: K as the MFMA A operand
+  // (key lq of each 16-key half, 8 dims per lane and step), V as 16-byte
+  // pieces for the transposed-read image; keys past the end read as zeros
+  auto load_tile = [&](int it, ushort8 (&kr)[2][STEPS], ushort8 (&vr)[NV]) {
     const bool pooled = it < pool_tiles;
     const int key_base =
         pooled ? it * WPM_KTILE : (tok_j0 + it - pool_tiles) * WPM_KTILE;
     const int key_end = pooled ? nb : pos + 1;
     const bf16* kc = pooled ? kp_cache : k_cache;
     const bf16* vc = pooled ? vp_cache : v_cache;
-    ushort8 vv[NV];
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int i = lane + WAVE_SIZE * j;
@@ -366,24 +368,41 @@ __global__ __launch_bounds__(256) void attn_window_pool_dec_kernel(
       if (key_base + key < key_end)
         v = *reinterpret_cast<const ushort8*>(
             vc + row_of(pooled, key_base + key) * V + col8);
-      vv[j] = v;
+      vr[j] = v;
     }
-    wp_f32x4 sc[2];
-    sc[0] = {0.f, 0.f, 0.f, 0.f};
-    sc[1] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub) {
       const int kg = key_base + sub * 16 + lq;
       const bool have = kg < key_end;
-      const bf16* kr = kc + (have ? row_of(pooled, kg) : 0) * D + 8 * la;
+      const bf16* krow = kc + (have ? row_of(pooled, kg) : 0) * D + 8 * la;
 #pragma unroll
       for (int st = 0; st < STEPS; ++st) {
         ushort8 u{};
-        if (have) u = *reinterpret_cast<const ushort8*>(kr + st * 32);
-        sc[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            *reinterpret_cast<wp_bf16x8*>(&u), qfrag[st], sc[sub], 0, 0, 0);
+        if (have) u = *reinterpret_cast<const ushort8*>(krow + st * 32);
+        kr[sub][st] = u;
       }
     }
+  };
+  ushort8 kreg[2][STEPS], vv[NV];
+  if (wave < n_iter) load_tile(wave, kreg, vv);
+
+  for (int it = wave; it < n_iter; it += 4) {
+    const bool pooled = it < pool_tiles;
+    const int key_base =
+        pooled ? it * WPM_KTILE : (tok_j0 + it - pool_tiles) * WPM_KTILE;
+    // the next tile's loads fly while this one computes
+    ushort8 knext[2][STEPS], vnext[NV];
+    if (it + 4 < n_iter) load_tile(it + 4, knext, vnext);
+    wp_f32x4 sc[2];
+    sc[0] = {0.f, 0.f, 0.f, 0.f};
+    sc[1] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int st = 0; st < STEPS; ++st)
+        sc[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            *reinterpret_cast<wp_bf16x8*>(&kreg[sub][st]), qfrag[st], sc[sub],
+            0, 0, 0);
     float p[8];
     float tile_max = -FLT_MAX;
 #pragma unroll
@@ -460,6 +479,14 @@ __global__ __launch_bounds__(256) void attn_window_pool_dec_kernel(
       }
       oacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
           *reinterpret_cast<wp_bf16x8*>(&pa), vb, oacc[c], 0, 0, 0);
+    }
+    if (it + 4 < n_iter) {
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st) kreg[sub][st] = knext[sub][st];
+#pragma unroll
+      for (int j = 0; j < NV; ++j) vv[j] = vnext[j];
     }
   }
 
