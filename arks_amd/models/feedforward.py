@@ -9,15 +9,16 @@ constants as constructor parameters:
   uses `top`; the router's softmax runs over all experts in fp32, experts
   form `groups` runs of neighbours and only those of the `keep` groups with
   the best single score can be chosen; the chosen scores are renormalised.
-  Expert weights are kept pre-transposed ([in, out]) like the framework's
-  other sparse feed-forward (models/llama_family.py MoEMLP); the gate|up
-  matrices of all experts sit side by side in ONE [width, experts * 2ff]
-  matrix. Two execution paths as there: up to DENSE_TOKENS rows every expert
-  runs on every row — one plain GEMM for all gate|up projections (no
-  per-expert copies of the rows), one batched GEMM down — with
-  data-independent shapes, so the step can be captured; above it the (row,
-  expert) pairs are sorted by expert and every expert runs plain GEMMs on
-  its own segment (its column block of the wide matrix).
+  The gate|up matrices of all experts are stacked in ONE [experts * 2ff,
+  width] matrix in the checkpoint's own [out, in] layout; the down matrices
+  are kept pre-transposed ([in, out] per expert) like the framework's other
+  sparse feed-forward (models/llama_family.py MoEMLP). Two execution paths
+  as there: up to DENSE_TOKENS rows every expert runs on every row — one
+  linear() for all gate|up projections (no per-expert copies of the rows),
+  one batched GEMM down — with data-independent shapes, so the step can be
+  captured; above it the (row, expert) pairs are sorted by expert and every
+  expert runs plain GEMMs on its own segment (its row block of the stacked
+  matrix).
 """
 
 from __future__ import annotations
@@ -58,16 +59,16 @@ class GroupedMoE(nn.Module):
         self.E, self.ff, self.top = experts, ff, top
         self.groups, self.keep, self.width = groups, keep, width
         self.router = _param(experts, width, dtype=dtype)
-        self.w13 = _param(width, experts * 2 * ff, dtype=dtype)
+        self.w13 = _param(experts * 2 * ff, width, dtype=dtype)
         self.w2 = _param(experts, ff, width, dtype=dtype)
 
     def weight_map(self) -> dict:
         m = {"router": (self.router, 0)}
         W, ff = self.width, self.ff
         for e in range(self.E):
+            m[f"e{e}.gate"] = (self.w13, e * 2 * ff, 0, (ff, W))
+            m[f"e{e}.up"] = (self.w13, e * 2 * ff + ff, 0, (ff, W))
             # (param, row, col, shape, expert index, transposed)
-            m[f"e{e}.gate"] = (self.w13, e * 2 * ff, 0, (ff, W), None, True)
-            m[f"e{e}.up"] = (self.w13, e * 2 * ff + ff, 0, (ff, W), None, True)
             m[f"e{e}.down"] = (self.w2, 0, 0, (W, ff), e, True)
         return m
 
@@ -77,7 +78,7 @@ class GroupedMoE(nn.Module):
         z = linear_f32(h, self.router)  # fp32 logits
         weights, ids = ops.moe_route_grouped(z, k, self.groups, self.keep)
         if T <= self.DENSE_TOKENS:
-            gu = torch.mm(h, self.w13)  # [T, E * 2ff]
+            gu = linear(h, self.w13)  # [T, E * 2ff]
             a = ops.glu_act(gu.view(T * E, 2 * ff), "swiglu")
             y = torch.bmm(a.view(T, E, ff).transpose(0, 1), self.w2)
             return ops.moe_mix_seq(y, weights, ids)
@@ -94,7 +95,7 @@ class GroupedMoE(nn.Module):
         for e, n in enumerate(counts):
             if n:
                 torch.mm(xs[at:at + n],
-                         self.w13[:, e * 2 * ff:(e + 1) * 2 * ff],
+                         self.w13[e * 2 * ff:(e + 1) * 2 * ff].t(),
                          out=gu[at:at + n])
             at += n
         a = ops.glu_act(gu, "swiglu")

@@ -122,11 +122,24 @@ __global__ __launch_bounds__(256) void lightning_combine_kernel(
   const int slot = slots[s];
   const float lam = decay[e / DV];
   float carry = (start > 0 && slot >= 0) ? state[(int64_t)slot * H * DV + se] : 0.f;
-  for (int k = chunk_off[s]; k < chunk_off[s + 1]; ++k) {
-    float* p = part + (int64_t)k * H * DV + e;
-    const float local = *p;
-    *p = carry;
-    carry = powf(lam, (float)chunk_rows[k]) * carry + local;
+  // the next chunk's value is loaded before this chunk's slot is rewritten,
+  // and decay^rows is evaluated again only when the row count changes
+  // (every chunk but a sequence's last has the same)
+  const int k0 = chunk_off[s], k1 = chunk_off[s + 1];
+  const int64_t stride = (int64_t)H * DV;
+  float nxt = k0 < k1 ? part[(int64_t)k0 * stride + e] : 0.f;
+  int pw_rows = -1;
+  float pw = 1.f;
+  for (int k = k0; k < k1; ++k) {
+    const float local = nxt;
+    if (k + 1 < k1) nxt = part[(int64_t)(k + 1) * stride + e];
+    const int rws = chunk_rows[k];
+    if (rws != pw_rows) {
+      pw = powf(lam, (float)rws);
+      pw_rows = rws;
+    }
+    part[(int64_t)k * stride + e] = carry;
+    carry = pw * carry + local;
   }
   if (slot >= 0) state[(int64_t)slot * H * DV + se] = carry;
 }
