@@ -499,11 +499,12 @@ def test_cli_flags_map_to_engine_config():
     assert cfg2.enable_prefix_caching is True
 
 
-def test_gagorax_preset_serves_completions():
+@pytest.mark.parametrize("preset", ["tiny-gagorax", "tiny-fusolix"])
+def test_layer_list_preset_serves_completions(preset):
     """A layer-list model (recurrent state slots, no prefix reuse) behind
     the same HTTP front: a completion and a streamed chat, twice, so slots
     and pages are taken and given back."""
-    cfg = EngineConfig(preset="tiny-gagorax", device="cpu", kv_cache_blocks=64,
+    cfg = EngineConfig(preset=preset, device="cpu", kv_cache_blocks=64,
                        max_model_len=256, max_num_seqs=2)
     engine = AsyncEngine(cfg, model_name="g")
     mc = cfg.model_config()
