@@ -7,8 +7,8 @@ constants as constructor parameters:
   act = g * sigmoid(alpha g) * (u + 1). Gate and up are one fused GEMM.
 - GroupedMoE: `experts` small silu-GLU feed-forwards of which every row
   uses `top`; the router's softmax runs over all experts in fp32, experts
-  form `groups` runs of neighbours and only those of the `keep` groups with
-  the best single score can be chosen; the chosen scores are renormalised.
+  are cut into `groups` contiguous runs and only the `keep` runs holding the
+  highest single scores stay eligible; the chosen scores are renormalised.
   The gate|up matrices of all experts are stacked in ONE [experts * 2ff,
   width] matrix in the checkpoint's own [out, in] layout; the down matrices
   are kept pre-transposed ([in, out] per expert) like the framework's other

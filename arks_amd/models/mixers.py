@@ -16,7 +16,7 @@ constructor parameters so that more than one design can use it:
 - RetentionMixer: the lightning recurrence on plain rows (nothing
   activated) with partial rotary on q and k, scaled keys, a per-head unit
   RMS of the output and a silu gate.
-- ParallelMixer: two of the above side by side on the same input, as ONE
+- ParallelMixer: two of the above fed the same input, as ONE
   in-projection GEMM and ONE out-projection GEMM over the concatenated
   (pre-scaled) head outputs.
 
@@ -368,7 +368,7 @@ class RetentionMixer(SplitMixer):
     """S <- decay_h S + k v^T, o = S^T q per head on plain projections: q
     and k turned by their position over their first rot_dims dims
     (half-split pairs unless interleaved), k times k_scale after that; each
-    head's o divided by its root mean square, times silu(gate). fp32 state
+    head's o scaled to unit RMS, times silu(gate). fp32 state
     [H, D, V] per sequence; runs the lightning kernels."""
 
     def __init__(self, width: int, heads: int, dim: int, vdim: int, decay,

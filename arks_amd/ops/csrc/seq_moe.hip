@@ -2,9 +2,9 @@
 // feed-forward (arks_amd/models/feedforward.py GroupedMoE), bf16 or float
 // rows.
 //
-//   moe_route_grouped  softmax over all E experts in fp32; experts form
-//       `groups` equal runs of neighbours, a group scores its best expert
-//       and only experts of the `keep` best groups can be chosen; the `top`
+//   moe_route_grouped  softmax over all E experts in fp32; experts are cut into
+//       `groups` contiguous runs of E/groups, a run's score is its highest
+//       expert score and only the `keep` highest-scoring runs stay eligible; the `top`
 //       largest scores among those, divided by their sum (+1e-20). Ties go
 //       to the lower index (groups and experts).
 //   moe_mix_rows  out[t] = sum_j w[t][j] * y[row(t, j)], row given, or
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(64) void moe_route_grouped_kernel(
     g_s[gI] = best;
   }
   __syncthreads();
-  // keep the best groups: `keep` argmax passes, the others' experts are
+  // the eligible runs: `keep` argmax passes, the others' experts are
   // marked unavailable (score -1)
   if (keep < groups) {
     for (int r = 0; r < keep; ++r) {

@@ -721,8 +721,8 @@ def retention_scan(q, k, v, decay, state, cu_seqlens, seq_lens, state_slots,
 
 
 def head_norm_gate(o, gate, eps, heads, out, out_scale=1.0):
-    """Each head's slice of o [T, heads*V] (fp32) divided by its root mean
-    square (eps inside the root, no weight), times silu(gate), times
+    """Each head's slice of o [T, heads*V] (fp32) scaled to unit RMS
+    (o * rsqrt(mean(o^2) + eps), no weight), times silu(gate), times
     out_scale, into out [T, heads*V] (may be a column slice)."""
     T = o.shape[0]
     of = o.float().view(T, heads, -1)
@@ -747,9 +747,9 @@ def glu_act(gu, kind, limit=0.0, alpha=1.0):
 
 
 def moe_route_grouped(logits, top, groups, keep):
-    """Softmax over all experts; experts form `groups` equal runs of
-    neighbours, a group scores its best expert, only experts of the `keep`
-    best groups can be chosen; the `top` largest scores among those, their
+    """Softmax over all experts; experts are cut into `groups`
+    contiguous runs of E/groups, a run's score is its highest expert score
+    and only the `keep` highest-scoring runs stay eligible; the `top` largest scores among those, their
     scores divided by their sum (+1e-20). Ties go to the lower index.
     logits [T, E] fp32 -> (weights [T, top] fp32, ids [T, top] int32)."""
     s = torch.softmax(logits.float(), -1)

@@ -508,9 +508,9 @@ def _rounded(t, dtype):
 
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("window,pool,plan", [
-    (8, 4, [37, 1, 1, 2, 30]), (96, 16, [130, 1, 70, 1]), (5, 24, [3, 50, 1, 1, 64]),
+    (8, 4, [37, 1, 1, 2, 30]), (72, 12, [130, 1, 70, 1]), (5, 24, [3, 50, 1, 1, 64]),
     (16, 5, [1] * 45), (1, 1, [20, 1, 9]), (33, 16, [200]),
-], ids=["w8p4", "w96p16", "w5p24", "w16p5-decode", "w1p1", "w33p16-whole"])
+], ids=["w8p4", "w72p12", "w5p24", "w16p5-decode", "w1p1", "w33p16-whole"])
 def test_window_pool_attention(device, dtype, window, pool, plan):
     dev = _dev(device)
     H, G, D, V = 4, 2, 16, 16
